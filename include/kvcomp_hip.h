@@ -1,0 +1,170 @@
+/*
+ * kvcomp_hip.h -- C ABI of libkvcomp_hip.so: KVComp's KV-cache codec and compressed decode-attention
+ * path for AMD MI355X (gfx950), written directly in HIP.
+ *
+ * The entry points below are what a binding of the reference's `kvcomp_cuda` operator module
+ * (kvcomp_cuda_extension/export_kvcomp.cpp:8-26, signatures in kvcomp_cuda_extension/kvcomp_cuda.pyi)
+ * needs: plain device/host pointers and sizes, no framework types.  Each declaration cites the
+ * reference interface it replaces (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - d_* pointers are device memory on the CURRENT HIP device, h_* pointers are host memory.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls are asynchronous
+ *     on that stream unless stated otherwise.
+ *   - Return value 0 = success; negative = error, with a message from kvc_last_error() (thread local).
+ *     The reference aborts the process on a failed check (include/utils.h:7-15); this library returns
+ *     an error instead so a host language can raise.
+ *   - Symbol tensors are uint8 [NB, BS, B, H, D] contiguous: `tokens` = NB*BS, `stride` = B*H*D bytes
+ *     per token (kvcomp_cuda_extension/src/kernels.cu:939,986).
+ *   - Tile geometry (kernels.cu:431-444, 503-519, include/kernels.h:12-19):
+ *       K tile = 64 tokens x head_dim channels of one (b,h); lane t <-> token      (head_dim <= 128;
+ *                the reference requires head_dim == 128)
+ *       V tile = 128 tokens x 64 adjacent flat channels;     lane t <-> channel
+ *   - Wire structs (include/kernels.h:25-42, include/huffman.h:13-22), little-endian:
+ *       block_info  {u32 offset; u16 byte_num; u16 pad}  8 B per tile
+ *       thread_info {u16 end_byte*8 + pad_bits}          2 B per lane stream
+ *       encode table entry {u32 code; u32 length}        8 B per symbol, index = symbol
+ *       decode tree node   {u8 is_leaf; i8 a; i8 b}      3 B
+ *     Tile payloads are laid out in tile order (the reference claims offsets with a global atomic in
+ *     arrival order, kernels.cu:472-479); every per-tile quantity is identical to the reference's.
+ */
+#ifndef KVCOMP_HIP_H
+#define KVCOMP_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* export_kvcomp.cpp:9-12 / include/kernels.h:12-19 */
+#define KVC_K_VEC_LEN 128
+#define KVC_K_VEC_PER_BLK 64
+#define KVC_V_VEC_LEN 128
+#define KVC_V_VEC_PER_BLK 64
+
+/* (min, scale) group descriptor of the quantizer: bit set = that dimension of [NB, BS, B, H, D] is
+ * reduced over (BS = 1, B = 2, H = 4, D = 8).  NB is never reduced. */
+#define KVC_MASK_K_BLOCK 0xF   /* models/cache/kvcomp_encode.py:10-13  BlockQuant dims [1,2,3,4] */
+#define KVC_MASK_V_TOKEN 0xE   /* models/cache/kvcomp_encode.py:10-13  TokenQuant dims [2,3,4]   */
+#define KVC_MASK_CHANNEL 0x1   /* utils/compute.py:140  ChannelQuant                             */
+#define KVC_MASK_SIM_TOKEN 0xC /* utils/compute.py:141  TokenQuant on [B,H,NB,BS,D]              */
+#define KVC_MASK_VECTOR 0x8    /* utils/compute.py:142  VectorQuant                              */
+#define KVC_MASK_SIM_BLOCK 0xD /* utils/compute.py:139  BlockQuant on [B,H,NB,BS,D]              */
+
+/* Decode-tree node formats accepted by the decoders. */
+#define KVC_TREE_I8 3          /* the reference's 3-byte node (<= 127 nodes, symbols <= 127)      */
+#define KVC_TREE_I16 5         /* {u8 is_leaf; i16 a; i16 b}: same walk, lifts both limits        */
+
+const char *kvc_last_error(void);
+int kvc_abi_version(void);
+
+/* ---- sizes: calculate_buffer_size (kernels.cu:893-917) --------------------------------------------
+ * out4 = {block_infos bytes, thread_infos bytes, idx_offset bytes (8), payload pre-allocation bytes}. */
+int kvc_calculate_buffer_size(int64_t tokens, int64_t stride, int is_k, int64_t head_num, int64_t head_dim,
+                              int64_t out4[4]);
+
+/* ---- codebook: build_codebook (src/huffman.cpp:99-157) --------------------------------------------
+ * kvc_histogram: 256-bin counts of n device symbols, ADDED into d_counts (int64[256], device).
+ * kvc_build_codebook_host: Huffman tree from counts (min-heap on frequency only, ties resolved exactly
+ *   as std::priority_queue / heapq do, src/huffman.cpp:34-96) -> shift (= smallest symbol), the encode
+ *   table (src/huffman.cpp:166-187) and the decode tree (src/huffman.cpp:229-252) as host bytes.
+ *   tree_format KVC_TREE_I8 reproduces the reference bytes and fails if they cannot represent the code
+ *   (> 127 nodes, symbol > 127, lone symbol); KVC_TREE_I16 always works for >= 2 symbols. */
+int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts, void *stream);
+int kvc_build_codebook_host(const int64_t *h_counts256, int tree_format, int *shift,
+                            uint8_t *h_encode_table, int64_t encode_cap, int64_t *encode_bytes,
+                            uint8_t *h_decode_tree, int64_t decode_cap, int64_t *decode_bytes);
+
+/* ---- encode: k_/v_entropy_encode_cuda_export (kernels.cu:919-1011) --------------------------------
+ * Writes block_infos (tiles*8 B), thread_infos (tiles*64*2 B) and the payload; *h_total_bytes receives
+ * the payload size (the reference returns encoded_data[:total]).  Synchronises the stream before
+ * returning, like the reference's cudaDeviceSynchronize.  d_idx_offset (8 B) receives
+ * {u32 tiles, u32 bytes} as in include/kernels.h:34-42.  block_info.offset = base_global_offset +
+ * offset inside this call's payload.  Fails if a tile payload exceeds 8191 B (thread_info is u16) or
+ * the payload exceeds encoded_cap. */
+int kvc_k_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride,
+                         const uint8_t *d_encode_table, int64_t encode_table_bytes,
+                         uint8_t *d_block_infos, uint8_t *d_thread_infos, uint8_t *d_idx_offset,
+                         uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
+                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes, void *stream);
+int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride,
+                         const uint8_t *d_encode_table, int64_t encode_table_bytes,
+                         uint8_t *d_block_infos, uint8_t *d_thread_infos, uint8_t *d_idx_offset,
+                         uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
+                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes, void *stream);
+
+/* ---- decode: k_/v_entropy_decode_cuda_export (kernels.cu:1013-1087) -------------------------------
+ * d_out uint8 [tokens, stride].  If elapsed_ms != NULL the kernel is bracketed by events, the call
+ * waits for it and stores the elapsed milliseconds (the reference's return value); otherwise the call
+ * is asynchronous. */
+int kvc_k_entropy_decode(const uint8_t *d_encoded, int64_t encoded_bytes,
+                         const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                         const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                         const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+                         uint8_t *d_out, int64_t tokens, int64_t stride,
+                         int64_t head_num, int64_t head_dim, float *elapsed_ms, void *stream);
+int kvc_v_entropy_decode(const uint8_t *d_encoded, int64_t encoded_bytes,
+                         const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                         const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                         const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+                         uint8_t *d_out, int64_t tokens, int64_t stride,
+                         int64_t head_num, int64_t head_dim, float *elapsed_ms, void *stream);
+
+/* ---- fused decode + matvec: k_/v_decode_and_mat_vec_mul_cuda_export (kernels.cu:1093-1180) --------
+ * K: d_q fp16 [batch, q_heads, head_dim]; d_scores fp16 [batch, q_heads, tokens]:
+ *      scores[b,hq,t] = sum_i dequant(K[t,b,hq/rep,i]) * q[b,hq,i]          (kernels.cu:721-776)
+ * V: d_p fp16 [batch, q_heads, tokens]; d_partial fp16 [tokens/128, batch, q_heads, head_dim]:
+ *      partial[g,b,hq,d] = sum_{t<128} dequant(V[128g+t,b,hq/rep,d]) * p[b,hq,128g+t]
+ *    (kernels.cu:778-861; the caller sums over g, models/cache/kvcomp_encode.py:275)
+ * quant_mask selects the (min, scale) layout: the reference's kernels take KVC_MASK_K_BLOCK for K
+ * (kernels.cu:771-772) and KVC_MASK_V_TOKEN for V (kernels.cu:822-833); K also accepts
+ * KVC_MASK_CHANNEL (min/scale per (block, b, h, channel)).  q_heads must be a multiple of kv_heads
+ * (the reference has q_heads == kv_heads).  Decoded symbols stay in registers; accumulation is fp32
+ * (the reference accumulates in fp16, kernels.cu:321,378).  elapsed_ms as for decode. */
+int kvc_k_decode_and_mat_vec_mul(const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+                                 const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                                 const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                                 const uint8_t *d_encoded, int64_t encoded_bytes,
+                                 const int8_t *d_quant_min_ints, const void *d_quant_scales_f16, int quant_mask,
+                                 const void *d_q_f16, void *d_scores_f16,
+                                 int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                                 float *elapsed_ms, void *stream);
+int kvc_v_decode_and_mat_vec_mul(const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+                                 const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                                 const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                                 const uint8_t *d_encoded, int64_t encoded_bytes,
+                                 const int8_t *d_quant_min_ints, const void *d_quant_scales_f16, int quant_mask,
+                                 const void *d_p_f16, void *d_partial_f16,
+                                 int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                                 float *elapsed_ms, void *stream);
+
+/* ---- dense baseline: k_mat_vec_mul_cuda_export (kernels.cu:1182-1273) ------------------------------
+ * d_k fp16 [tokens, batch, heads, head_dim], d_q fp16 [batch, heads, head_dim],
+ * d_out fp16 [tokens, batch, heads].  (The reference requires batch == 1 and head_dim == 128.) */
+int kvc_k_mat_vec_mul(const void *d_k_f16, const void *d_q_f16, void *d_out_f16,
+                      int64_t tokens, int64_t batch, int64_t heads, int64_t head_dim,
+                      float *elapsed_ms, void *stream);
+
+/* ---- quantizer: quant (utils/compute.py:93-106; src/compute.cpp:40-58) and quant_ints (:74-91) -----
+ * d_x fp16 [NB, BS, B, H, D]; groups given by quant_mask.  Bit-exact with the reference's chain of
+ * fp16 PyTorch ops: scale = RN16(f32(RN16(max-min)) * eb); min_i = rint(RN16(min/scale));
+ * sym = RN16(rint(RN16(x/scale)) - min_i).  Outputs: d_sym uint8 (same shape), d_min_i8 int8[groups],
+ * d_scale_f16 fp16[groups] (the casts of models/cache/kvcomp_encode.py:97-98); optional fp16 copies
+ * d_min_f16 (may be NULL).  Optionally accumulates the 256-bin symbol histogram into d_counts
+ * (int64[256], may be NULL). */
+int64_t kvc_quant_groups(int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask);
+int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+              float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
+              int64_t *d_counts, void *stream);
+
+/* ---- dequantizer: (sym + min_i) * scale (models/cache/kvcomp_encode.py:146,161) --------------------
+ * d_out fp16 = RN16(f32(sym + min_i) * f32(scale)), same shape as d_sym. */
+int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const void *d_scale_f16,
+                int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                void *d_out_f16, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KVCOMP_HIP_H */

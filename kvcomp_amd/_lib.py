@@ -1,0 +1,63 @@
+"""ctypes binding of kvcomp_amd/lib/libkvcomp_hip.so (the C ABI of include/kvcomp_hip.h).
+
+There is no CPU fallback: if the library is missing or a call fails, an exception is raised.
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libkvcomp_hip.so")
+_LIB = None
+
+_i64, _int, _vp, _f32p, _u32 = C.c_int64, C.c_int, C.c_void_p, C.POINTER(C.c_float), C.c_uint32
+_i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
+
+# name -> argtypes (every function returns int unless listed in _RESTYPES)
+_SIGNATURES = {
+    "kvc_abi_version": [],
+    "kvc_calculate_buffer_size": [_i64, _i64, _int, _i64, _i64, _i64p],
+    "kvc_histogram": [_vp, _i64, _vp, _vp],
+    "kvc_build_codebook_host": [_i64p, _int, _intp, _vp, _i64, _i64p, _vp, _i64, _i64p],
+    "kvc_k_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _vp],
+    "kvc_v_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _vp],
+    "kvc_k_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_v_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_k_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,
+                                     _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_v_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,
+                                     _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_k_mat_vec_mul": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_quant_groups": [_i64, _i64, _i64, _i64, _i64, _int],
+    "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],
+    "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
+}
+_RESTYPES = {"kvc_quant_groups": _i64}
+
+EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["kvc_last_error"])
+
+
+class KvcompError(RuntimeError):
+    pass
+
+
+def lib():
+    """Load the shared library (once).  Raises if it has not been built: there is no other code path."""
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise KvcompError("%s is missing: build it with `python -m kvcomp_amd.build` "
+                              "(this package has no CPU fallback)" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        L.kvc_last_error.restype = C.c_char_p
+        L.kvc_last_error.argtypes = []
+        for name, args in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.argtypes = args
+            fn.restype = _RESTYPES.get(name, _int)
+        _LIB = L
+    return _LIB
+
+
+def check(rc):
+    if rc != 0:
+        raise KvcompError(lib().kvc_last_error().decode("utf-8", "replace") or "libkvcomp_hip call failed (%d)" % rc)

@@ -1,0 +1,116 @@
+// kvc_common.h -- shared host/device definitions of libkvcomp_hip (gfx950, wave64).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+#include <stdarg.h>
+
+#include "../../include/kvcomp_hip.h"
+
+// ---------------------------------------------------------------------------------------------------
+// geometry
+// ---------------------------------------------------------------------------------------------------
+constexpr int KVC_WAVE = 64;               // lanes per tile = vectors per tile (include/kernels.h:13,18)
+constexpr int KVC_WAVES_PER_WG = 4;
+constexpr int KVC_WG = KVC_WAVE * KVC_WAVES_PER_WG;
+constexpr int KVC_V_TOKENS = 128;          // tokens per V vector (include/kernels.h:17)
+constexpr int KVC_MAX_TILE_BYTES = 8191;   // thread_info is u16 = end_byte*8 + pad (include/kernels.h:30-32)
+
+// Payload staging area of one wave in LDS: the tile payload plus the up-to-15 bytes that precede it
+// in its first 16-byte chunk, rounded up, plus two guard words for the look-ahead of the last refill.
+constexpr int KVC_STAGE_BYTES = ((KVC_MAX_TILE_BYTES + 15 + 15) / 16) * 16 + 16;   // 8224
+constexpr int KVC_STAGE_WORDS = KVC_STAGE_BYTES / 4;
+
+// ---------------------------------------------------------------------------------------------------
+// decode look-up table (built on the device from the decode tree, see kvc_lut.hip)
+//
+//   header   {lbits, lmax, n_long, group}
+//   long[ ]  codes longer than lbits: {code left-aligned in 32 bits, len | sym << 8}
+//   entry[ ] 1 << lbits words indexed by the next lbits stream bits: len | sym << 8, or 0 when the
+//            code is longer than lbits (search long[]) or the bits match no code.
+//   group    how many symbols may be decoded from one 32-bit window: floor(32 / lmax), one of 8,4,2,1.
+// ---------------------------------------------------------------------------------------------------
+constexpr int KVC_LUT_MAX_BITS = 10;
+constexpr int KVC_LUT_MAX_LONG = 256;
+constexpr int KVC_LUT_HEADER_WORDS = 4;
+constexpr int KVC_LUT_LONG_WORDS = 2 * KVC_LUT_MAX_LONG;
+constexpr int KVC_LUT_ENTRY_WORDS = 1 << KVC_LUT_MAX_BITS;
+constexpr int KVC_LUT_WORDS = KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS + KVC_LUT_ENTRY_WORDS;
+constexpr int KVC_LUT_BYTES = KVC_LUT_WORDS * 4;          // 6160
+constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2, rounded up
+
+// ---------------------------------------------------------------------------------------------------
+// host helpers (kvc_host.hip)
+// ---------------------------------------------------------------------------------------------------
+int kvc_fail(int code, const char *fmt, ...);
+int kvc_check_hip(hipError_t e, const char *what);
+// A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the
+// reference-signature entry points derive from the decode tree on every call.
+constexpr size_t KVC_WS_SLOT_BYTES = 16384;
+int kvc_workspace_slot(void **slot);
+int kvc_launch_build_lut(const uint8_t *d_tree, int64_t tree_bytes, int tree_format, uint32_t *d_lut,
+                         int n_codebooks, int64_t tree_stride_bytes, hipStream_t stream);
+
+#define KVC_REQUIRE(cond, ...)                     \
+    do {                                           \
+        if (!(cond)) return kvc_fail(-1, __VA_ARGS__); \
+    } while (0)
+#define KVC_HIP(call)                              \
+    do {                                           \
+        int rc_ = kvc_check_hip((call), #call);    \
+        if (rc_) return rc_;                       \
+    } while (0)
+
+// Optional event bracket implementing the reference's "returns elapsed milliseconds" contract
+// (kvcomp_cuda_extension/src/kernels.cu:1026-1048).
+struct KvcTimer {
+    hipEvent_t a = nullptr, b = nullptr;
+    hipStream_t s;
+    float *out;
+    KvcTimer(float *out_, hipStream_t s_) : s(s_), out(out_) {
+        if (out) {
+            (void)hipEventCreate(&a);
+            (void)hipEventCreate(&b);
+            (void)hipEventRecord(a, s);
+        }
+    }
+    int finish() {
+        if (!out) return 0;
+        hipError_t e = hipEventRecord(b, s);
+        if (e == hipSuccess) e = hipEventSynchronize(b);
+        if (e == hipSuccess) e = hipEventElapsedTime(out, a, b);
+        (void)hipEventDestroy(a);
+        (void)hipEventDestroy(b);
+        return kvc_check_hip(e, "event timing");
+    }
+};
+
+// ---------------------------------------------------------------------------------------------------
+// device helpers
+// ---------------------------------------------------------------------------------------------------
+#ifdef __HIPCC__
+__device__ __forceinline__ uint32_t kvc_bswap(uint32_t v) { return __builtin_bswap32(v); }
+
+__device__ __forceinline__ float kvc_readlane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+
+__device__ __forceinline__ float kvc_wave_sum(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// inclusive prefix sum over the 64 lanes of a wave
+__device__ __forceinline__ uint32_t kvc_wave_inclusive_scan(uint32_t v, int lane)
+{
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        uint32_t t = __shfl_up(v, off, 64);
+        if (lane >= off) v += t;
+    }
+    return v;
+}
+#endif

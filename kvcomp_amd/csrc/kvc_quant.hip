@@ -1,0 +1,391 @@
+// kvc_quant.hip -- error-bounded block quantizer, dequantizer, symbol histogram and the dense matvec
+// baseline.
+//
+//   kvc_quant      <- quant (utils/compute.py:93-106, src/compute.cpp:40-58) and quant_ints
+//                     (utils/compute.py:74-91), which the reference runs as ~8 separate fp16 PyTorch
+//                     kernels; here: min/max by wavefront reductions, then one pass that writes symbols.
+//   kvc_dequant    <- (sym + min_i) * scale (models/cache/kvcomp_encode.py:146,161)
+//   kvc_histogram  <- torch::bincount in build_codebook (src/huffman.cpp:105-109), with LDS atomics
+//   kvc_k_mat_vec_mul <- k_mat_vec_mul (src/kernels.cu:1192-1273)
+//
+// Bit-exactness of the quantizer: every reference op is an fp16 tensor op, i.e. an fp32 operation on
+// the exact fp16 inputs followed by one rounding to fp16.  The device code spells out exactly that
+// chain; the fp32 division is IEEE (correctly rounded) and fp16/fp32 subnormals are kept.
+#include "kvc_common.h"
+
+// ---------------------------------------------------------------------------------------------------
+// scalar pieces of the reference arithmetic
+// ---------------------------------------------------------------------------------------------------
+struct KvcGroupParams {
+    float scale;     // exact value of the fp16 scale
+    float min_i;     // exact value of the fp16 rounded min / scale
+    __half scale_h, min_h;
+};
+
+__device__ __forceinline__ KvcGroupParams kvc_group_params(float mn, float mx, float eb)
+{
+    KvcGroupParams g;
+    const __half range = __float2half_rn(mx - mn);                          // (max_ - min_)
+    g.scale_h = __float2half_rn(__half2float(range) * eb);                  // * quant_scale_rel
+    g.scale = __half2float(g.scale_h);
+    const __half mq = __float2half_rn(__fdiv_rn(mn, g.scale));              // min_ / quant_scale
+    g.min_h = __float2half_rn(rintf(__half2float(mq)));                     // .round_()
+    g.min_i = __half2float(g.min_h);
+    return g;
+}
+
+__device__ __forceinline__ uint8_t kvc_quant_one(float x, const KvcGroupParams &g)
+{
+    const __half q = __float2half_rn(__fdiv_rn(x, g.scale));                // tensor / quant_scale
+    const float qi = __half2float(__float2half_rn(rintf(__half2float(q)))); // .round_()
+    const __half s = __float2half_rn(qi - g.min_i);                         // quant_ints - min_ints
+    return (uint8_t)(int)__half2float(s);                                   // .to(torch.uint8)
+}
+
+__device__ __forceinline__ float kvc_wave_min(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fminf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float kvc_wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// order-preserving float <-> uint map for atomicMin / atomicMax
+__device__ __forceinline__ uint32_t kvc_f2ord(float f)
+{
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float kvc_ord2f(uint32_t o)
+{
+    return __uint_as_float((o & 0x80000000u) ? (o & 0x7fffffffu) : ~o);
+}
+
+struct KvcQuantArgs {
+    const __half *x;
+    int64_t NB, BS, B, H, D;
+    int mask;
+    float eb;
+    uint8_t *sym;
+    int8_t *min_i8;
+    __half *scale_f16;
+    __half *min_f16;       // optional
+    uint32_t *minmax;      // block modes: {ord(min), ord(max)} per group
+};
+
+// ---- per-channel groups (mask 0x1): a thread owns two adjacent channels of one block and walks the
+// BS tokens twice; no cross-lane traffic at all. ------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_kernel(KvcQuantArgs a)
+{
+    const int64_t stride = a.B * a.H * a.D;
+    const int64_t pairs = stride >> 1;
+    const int64_t gid = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
+    if (gid >= a.NB * pairs) return;
+    const int64_t nb = gid / pairs, c = (gid - nb * pairs) * 2;
+    const __half *p = a.x + nb * a.BS * stride + c;
+    float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+    for (int64_t t = 0; t < a.BS; t++) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + t * stride);
+        const float v0 = __low2float(v), v1 = __high2float(v);
+        mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
+        mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
+    }
+    const KvcGroupParams g0 = kvc_group_params(mn0, mx0, a.eb), g1 = kvc_group_params(mn1, mx1, a.eb);
+    const int64_t g = nb * stride + c;
+    a.scale_f16[g] = g0.scale_h;
+    a.scale_f16[g + 1] = g1.scale_h;
+    a.min_i8[g] = (int8_t)(int)g0.min_i;
+    a.min_i8[g + 1] = (int8_t)(int)g1.min_i;
+    if (a.min_f16) { a.min_f16[g] = g0.min_h; a.min_f16[g + 1] = g1.min_h; }
+    uint8_t *s = a.sym + nb * a.BS * stride + c;
+    for (int64_t t = 0; t < a.BS; t++) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + t * stride);
+        uchar2 o;
+        o.x = kvc_quant_one(__low2float(v), g0);
+        o.y = kvc_quant_one(__high2float(v), g1);
+        *reinterpret_cast<uchar2 *>(s + t * stride) = o;
+    }
+}
+
+// ---- row groups (masks 0xE, 0xC, 0x8): a group is one contiguous run of R elements; one wave per
+// group, min/max by wavefront reduction. -------------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, int64_t R, int64_t groups)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
+    if (g >= groups) return;
+    const __half *p = a.x + g * R;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+        const float v0 = __low2float(v), v1 = __high2float(v);
+        mn = fminf(mn, fminf(v0, v1));
+        mx = fmaxf(mx, fmaxf(v0, v1));
+    }
+    mn = kvc_wave_min(mn);
+    mx = kvc_wave_max(mx);
+    const KvcGroupParams gp = kvc_group_params(mn, mx, a.eb);
+    if (lane == 0) {
+        a.scale_f16[g] = gp.scale_h;
+        a.min_i8[g] = (int8_t)(int)gp.min_i;
+        if (a.min_f16) a.min_f16[g] = gp.min_h;
+    }
+    uint8_t *s = a.sym + g * R;
+    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+        uchar2 o;
+        o.x = kvc_quant_one(__low2float(v), gp);
+        o.y = kvc_quant_one(__high2float(v), gp);
+        *reinterpret_cast<uchar2 *>(s + i) = o;
+    }
+}
+
+// ---- block groups (masks 0xF, 0xD): rows of R contiguous elements map many-to-one onto groups;
+// wave-reduce each row, then merge rows with atomics on an order-preserving integer image. -----------
+__device__ __forceinline__ int64_t kvc_block_group_of_row(const KvcQuantArgs &a, int64_t row)
+{
+    if (a.mask == KVC_MASK_K_BLOCK) return row / a.BS;                 // row = token
+    const int64_t b = row % a.B;                                       // row = (token, b)
+    return (row / (a.BS * a.B)) * a.B + b;
+}
+
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_block_init_kernel(uint32_t *minmax, int64_t groups)
+{
+    const int64_t g = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
+    if (g < groups) { minmax[2 * g] = 0xffffffffu; minmax[2 * g + 1] = 0u; }
+}
+
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_block_minmax_kernel(KvcQuantArgs a, int64_t R, int64_t rows)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const __half *p = a.x + row * R;
+    float mn = INFINITY, mx = -INFINITY;
+    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+        const float v0 = __low2float(v), v1 = __high2float(v);
+        mn = fminf(mn, fminf(v0, v1));
+        mx = fmaxf(mx, fmaxf(v0, v1));
+    }
+    mn = kvc_wave_min(mn);
+    mx = kvc_wave_max(mx);
+    if (lane == 0) {
+        const int64_t g = kvc_block_group_of_row(a, row);
+        atomicMin(&a.minmax[2 * g], kvc_f2ord(mn));
+        atomicMax(&a.minmax[2 * g + 1], kvc_f2ord(mx));
+    }
+}
+
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_block_apply_kernel(KvcQuantArgs a, int64_t R, int64_t rows)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t g = kvc_block_group_of_row(a, row);
+    const KvcGroupParams gp = kvc_group_params(kvc_ord2f(a.minmax[2 * g]), kvc_ord2f(a.minmax[2 * g + 1]), a.eb);
+    // the first row of a group also publishes the group's metadata
+    const bool first = a.mask == KVC_MASK_K_BLOCK ? (row % a.BS == 0) : ((row / a.B) % a.BS == 0);
+    if (first && lane == 0) {
+        a.scale_f16[g] = gp.scale_h;
+        a.min_i8[g] = (int8_t)(int)gp.min_i;
+        if (a.min_f16) a.min_f16[g] = gp.min_h;
+    }
+    const __half *p = a.x + row * R;
+    uint8_t *s = a.sym + row * R;
+    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+        uchar2 o;
+        o.x = kvc_quant_one(__low2float(v), gp);
+        o.y = kvc_quant_one(__high2float(v), gp);
+        *reinterpret_cast<uchar2 *>(s + i) = o;
+    }
+}
+
+extern "C" int64_t kvc_quant_groups(int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int mask)
+{
+    return NB * ((mask & 1) ? 1 : BS) * ((mask & 2) ? 1 : B) * ((mask & 4) ? 1 : H) * ((mask & 8) ? 1 : D);
+}
+
+extern "C" int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts, void *stream);
+
+extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                         float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
+                         int64_t *d_counts, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    KVC_REQUIRE(NB >= 0 && BS > 0 && B > 0 && H > 0 && D > 0, "bad shape");
+    KVC_REQUIRE(D % 2 == 0, "head_dim must be even");
+    KVC_REQUIRE(((uintptr_t)d_x_f16 & 3) == 0 && ((uintptr_t)d_sym & 1) == 0, "quantizer buffers are misaligned");
+    KVC_REQUIRE(eb > 0.f, "error bound must be positive");
+    if (NB == 0) return 0;
+    KvcQuantArgs a;
+    a.x = reinterpret_cast<const __half *>(d_x_f16);
+    a.NB = NB; a.BS = BS; a.B = B; a.H = H; a.D = D;
+    a.mask = quant_mask;
+    a.eb = eb;
+    a.sym = d_sym;
+    a.min_i8 = d_min_i8;
+    a.scale_f16 = reinterpret_cast<__half *>(d_scale_f16);
+    a.min_f16 = reinterpret_cast<__half *>(d_min_f16);
+    a.minmax = nullptr;
+    const int64_t stride = B * H * D;
+    if (quant_mask == KVC_MASK_CHANNEL) {
+        const int64_t threads = NB * (stride / 2);
+        hipLaunchKernelGGL(kvc_quant_channel_kernel, dim3((unsigned)((threads + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a);
+    } else if (quant_mask == KVC_MASK_V_TOKEN || quant_mask == KVC_MASK_SIM_TOKEN || quant_mask == KVC_MASK_VECTOR) {
+        const int64_t R = quant_mask == KVC_MASK_V_TOKEN ? stride : quant_mask == KVC_MASK_SIM_TOKEN ? H * D : D;
+        const int64_t groups = NB * BS * stride / R;
+        hipLaunchKernelGGL(kvc_quant_row_kernel, dim3((unsigned)((groups + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG)),
+                           dim3(KVC_WG), 0, stream, a, R, groups);
+    } else if (quant_mask == KVC_MASK_K_BLOCK || quant_mask == KVC_MASK_SIM_BLOCK) {
+        const int64_t R = quant_mask == KVC_MASK_K_BLOCK ? stride : H * D;
+        const int64_t rows = NB * BS * stride / R;
+        const int64_t groups = quant_mask == KVC_MASK_K_BLOCK ? NB : NB * B;
+        KVC_REQUIRE(groups * 8 <= (int64_t)KVC_WS_SLOT_BYTES, "too many block-quantization groups (%lld) for one call", (long long)groups);
+        void *slot;
+        if (int rc = kvc_workspace_slot(&slot)) return rc;
+        a.minmax = reinterpret_cast<uint32_t *>(slot);
+        const unsigned row_wgs = (unsigned)((rows + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
+        hipLaunchKernelGGL(kvc_quant_block_init_kernel, dim3((unsigned)((groups + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a.minmax, groups);
+        hipLaunchKernelGGL(kvc_quant_block_minmax_kernel, dim3(row_wgs), dim3(KVC_WG), 0, stream, a, R, rows);
+        hipLaunchKernelGGL(kvc_quant_block_apply_kernel, dim3(row_wgs), dim3(KVC_WG), 0, stream, a, R, rows);
+    } else {
+        return kvc_fail(-1, "unsupported quantization group mask 0x%x", quant_mask);
+    }
+    KVC_HIP(hipGetLastError());
+    if (d_counts) return kvc_histogram(d_sym, NB * BS * stride, d_counts, stream_);
+    return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// dequantizer
+// ---------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_dequant_kernel(const uint8_t *__restrict__ sym, const int8_t *__restrict__ min_i8,
+                                                             const __half *__restrict__ scale, int64_t BS, int64_t B, int64_t H,
+                                                             int64_t D, int mask, __half *__restrict__ out, int64_t n)
+{
+    const int64_t gBS = (mask & 1) ? 1 : BS, gB = (mask & 2) ? 1 : B, gH = (mask & 4) ? 1 : H, gD = (mask & 8) ? 1 : D;
+    for (int64_t i = (int64_t)blockIdx.x * KVC_WG + threadIdx.x; i < n; i += (int64_t)gridDim.x * KVC_WG) {
+        int64_t r = i;
+        const int64_t d = r % D; r /= D;
+        const int64_t h = r % H; r /= H;
+        const int64_t b = r % B; r /= B;
+        const int64_t bs = r % BS;
+        const int64_t nb = r / BS;
+        const int64_t g = (((nb * gBS + ((mask & 1) ? 0 : bs)) * gB + ((mask & 2) ? 0 : b)) * gH + ((mask & 4) ? 0 : h)) * gD +
+                          ((mask & 8) ? 0 : d);
+        const int v = (int)sym[i] + (int)min_i8[g];
+        out[i] = __float2half_rn((float)v * __half2float(scale[g]));
+    }
+}
+
+extern "C" int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const void *d_scale_f16, int64_t NB, int64_t BS,
+                           int64_t B, int64_t H, int64_t D, int quant_mask, void *d_out_f16, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    KVC_REQUIRE(NB >= 0 && BS > 0 && B > 0 && H > 0 && D > 0, "bad shape");
+    KVC_REQUIRE((quant_mask & ~0xF) == 0, "bad quantization group mask");
+    const int64_t n = NB * BS * B * H * D;
+    if (n == 0) return 0;
+    int64_t wgs = (n + KVC_WG - 1) / KVC_WG;
+    if (wgs > 65536) wgs = 65536;
+    hipLaunchKernelGGL(kvc_dequant_kernel, dim3((unsigned)wgs), dim3(KVC_WG), 0, stream, d_sym, d_min_i8,
+                       reinterpret_cast<const __half *>(d_scale_f16), BS, B, H, D, quant_mask,
+                       reinterpret_cast<__half *>(d_out_f16), n);
+    return kvc_check_hip(hipGetLastError(), "kvc_dequant_kernel launch");
+}
+
+// ---------------------------------------------------------------------------------------------------
+// histogram
+// ---------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_histogram_kernel(const uint8_t *__restrict__ sym, int64_t n,
+                                                               unsigned long long *__restrict__ counts)
+{
+    __shared__ uint32_t s_bins[KVC_WAVES_PER_WG][256];   // one copy per wave: fewer same-address collisions
+    const int tid = threadIdx.x, wave = tid >> 6;
+    for (int i = tid; i < KVC_WAVES_PER_WG * 256; i += KVC_WG) (&s_bins[0][0])[i] = 0;
+    __syncthreads();
+    const int64_t nwords = n >> 2;
+    const uint32_t *w = reinterpret_cast<const uint32_t *>(sym);
+    for (int64_t i = (int64_t)blockIdx.x * KVC_WG + tid; i < nwords; i += (int64_t)gridDim.x * KVC_WG) {
+        const uint32_t v = w[i];
+        atomicAdd(&s_bins[wave][v & 0xffu], 1u);
+        atomicAdd(&s_bins[wave][(v >> 8) & 0xffu], 1u);
+        atomicAdd(&s_bins[wave][(v >> 16) & 0xffu], 1u);
+        atomicAdd(&s_bins[wave][v >> 24], 1u);
+    }
+    if (blockIdx.x == 0 && tid < (int)(n & 3)) atomicAdd(&s_bins[0][sym[(nwords << 2) + tid]], 1u);
+    __syncthreads();
+    uint32_t c = 0;
+#pragma unroll
+    for (int k = 0; k < KVC_WAVES_PER_WG; k++) c += s_bins[k][tid];
+    if (c) atomicAdd(&counts[tid], (unsigned long long)c);
+}
+
+extern "C" int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    KVC_REQUIRE(n >= 0, "negative length");
+    KVC_REQUIRE(((uintptr_t)d_sym & 3) == 0, "symbol pointer must be 4-byte aligned");
+    if (n == 0) return 0;
+    int64_t wgs = (n / 4 + KVC_WG * 16 - 1) / (KVC_WG * 16);   // ~64 symbols per thread, 2^32 per workgroup at most
+    if (wgs < 1) wgs = 1;
+    if (wgs > 4096) wgs = 4096;
+    KVC_REQUIRE(n / wgs < (1ll << 31), "input too large for 32-bit workgroup counters");
+    hipLaunchKernelGGL(kvc_histogram_kernel, dim3((unsigned)wgs), dim3(KVC_WG), 0, stream, d_sym, n,
+                       reinterpret_cast<unsigned long long *>(d_counts));
+    return kvc_check_hip(hipGetLastError(), "kvc_histogram_kernel launch");
+}
+
+// ---------------------------------------------------------------------------------------------------
+// dense matvec baseline: out[t,b,h] = sum_i k[t,b,h,i] * q[b,h,i], fp32 accumulation.
+// A row of head_dim halves is read by head_dim/8 adjacent lanes with 16-byte loads.
+// ---------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_k_mat_vec_mul_kernel(const __half *__restrict__ k, const __half *__restrict__ q,
+                                                                   __half *__restrict__ out, int64_t rows, int bh, int D)
+{
+    const int lpr = D >> 3;                    // lanes per row (power of two, <= 16)
+    const int rpw = KVC_WG / lpr;              // rows per workgroup pass
+    const int sub = threadIdx.x % lpr;
+    for (int64_t row = (int64_t)blockIdx.x * rpw + threadIdx.x / lpr; row < rows; row += (int64_t)gridDim.x * rpw) {
+        const uint4 kv = *reinterpret_cast<const uint4 *>(k + row * D + sub * 8);
+        const uint4 qv = *reinterpret_cast<const uint4 *>(q + (row % bh) * D + sub * 8);
+        const __half2 *kh = reinterpret_cast<const __half2 *>(&kv), *qh = reinterpret_cast<const __half2 *>(&qv);
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            acc = fmaf(__low2float(kh[j]), __low2float(qh[j]), acc);
+            acc = fmaf(__high2float(kh[j]), __high2float(qh[j]), acc);
+        }
+        for (int off = lpr >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (sub == 0) out[row] = __float2half_rn(acc);
+    }
+}
+
+extern "C" int kvc_k_mat_vec_mul(const void *d_k_f16, const void *d_q_f16, void *d_out_f16, int64_t tokens, int64_t batch,
+                                 int64_t heads, int64_t head_dim, float *elapsed_ms, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    KVC_REQUIRE(head_dim == 16 || head_dim == 32 || head_dim == 64 || head_dim == 128, "head_dim must be 16, 32, 64 or 128");
+    KVC_REQUIRE(((uintptr_t)d_k_f16 & 15) == 0 && ((uintptr_t)d_q_f16 & 15) == 0, "k and q must be 16-byte aligned");
+    const int64_t rows = tokens * batch * heads;
+    if (rows == 0) {
+        if (elapsed_ms) *elapsed_ms = 0.f;
+        return 0;
+    }
+    const int rpw = KVC_WG / (int)(head_dim / 8);
+    int64_t wgs = (rows + rpw - 1) / rpw;
+    if (wgs > 16384) wgs = 16384;
+    KvcTimer timer(elapsed_ms, stream);
+    hipLaunchKernelGGL(kvc_k_mat_vec_mul_kernel, dim3((unsigned)wgs), dim3(KVC_WG), 0, stream,
+                       reinterpret_cast<const __half *>(d_k_f16), reinterpret_cast<const __half *>(d_q_f16),
+                       reinterpret_cast<__half *>(d_out_f16), rows, (int)(batch * heads), (int)head_dim);
+    KVC_HIP(hipGetLastError());
+    return timer.finish();
+}

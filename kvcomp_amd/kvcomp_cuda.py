@@ -1,0 +1,240 @@
+"""Drop-in mirror of the reference's `kvcomp_cuda` operator module for AMD MI355X.
+
+Same names, argument order and meaning as kvcomp_cuda_extension/kvcomp_cuda.pyi:14-84 and
+kvcomp_cuda_extension/export_kvcomp.cpp:8-26 (4 constants + 9 functions); every call goes through the C
+ABI of libkvcomp_hip.so (include/kvcomp_hip.h) on torch's current stream.  To make the reference's own
+callers pick it up:
+
+    import sys, kvcomp_amd.kvcomp_cuda as m; sys.modules["kvcomp_cuda"] = m
+
+Differences from the reference, all deliberate:
+  * failed checks raise KvcompError (a RuntimeError) instead of aborting the process
+    (include/utils.h:7-15);
+  * tile payloads are laid out in tile order, not in the arrival order of a global atomic
+    (src/kernels.cu:472-479) -- per-tile bytes, thread_infos and byte counts are identical;
+  * batch > 1, head_dim < 128 (multiples of 8), grouped-query heads (B/q has more heads than head_num)
+    and per-channel K scales are accepted where the reference asserts or silently misbehaves;
+  * kernels run on torch's current stream rather than the legacy default stream.
+"""
+import ctypes as C
+from typing import List, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import KvcompError, check  # noqa: F401
+
+# export_kvcomp.cpp:9-12
+K_VEC_LEN = 128
+K_VEC_PER_BLK = 64
+V_VEC_LEN = 128
+V_VEC_PER_BLK = 64
+
+MASK_K_BLOCK, MASK_V_TOKEN, MASK_CHANNEL, MASK_SIM_TOKEN, MASK_VECTOR, MASK_SIM_BLOCK = 0xF, 0xE, 0x1, 0xC, 0x8, 0xD
+TREE_I8, TREE_I16 = 3, 5
+
+
+def _ptr(t: torch.Tensor):
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require(cond, msg):
+    if not cond:
+        raise KvcompError(msg)
+
+
+def _dev_u8(t, name):
+    _require(t.is_cuda, "%s must be a device tensor" % name)
+    _require(t.dtype == torch.uint8, "%s must be uint8" % name)
+    _require(t.is_contiguous(), "%s must be contiguous" % name)
+
+
+def _geometry(t5: torch.Tensor):
+    _require(t5.dim() == 5, "symbol tensor must be [NB, BS, B, H, D]")
+    tokens = t5.shape[0] * t5.shape[1]
+    stride = t5.shape[2] * t5.shape[3] * t5.shape[4]
+    return tokens, stride
+
+
+def calculate_buffer_size(input: torch.Tensor, is_k: bool, head_num: int, head_dim: int) -> Tuple[int, int, int, int]:
+    """src/kernels.cu:893-917: (block_infos, thread_infos, idx_offset, payload pre-allocation) in bytes."""
+    tokens, stride = _geometry(input)
+    out = (C.c_int64 * 4)()
+    check(_lib.lib().kvc_calculate_buffer_size(tokens, stride, int(bool(is_k)), head_num, head_dim, out))
+    return tuple(int(v) for v in out)
+
+
+def build_codebook(input_tensors: List[torch.Tensor], tree_format: int = TREE_I8) -> Tuple[int, torch.Tensor, torch.Tensor]:
+    """src/huffman.cpp:99-157: histogram of all inputs -> (shift, encode table, decode tree) as CPU uint8
+    tensors.  The histogram runs on the device the inputs live on (one 2 KiB copy back, where the
+    reference issues 256 .item() reads, huffman.cpp:42)."""
+    _require(len(input_tensors) > 0, "input_tensors must not be empty")
+    dev = input_tensors[0].device
+    for t in input_tensors:
+        _require(t.device == dev, "All input tensors must be on the same device.")
+        _require(t.dtype == torch.uint8, "Input tensors must be of type uint8.")
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        counts = torch.zeros(256, dtype=torch.int64, device=dev)
+        for t in input_tensors:
+            t = t.contiguous()
+            check(L.kvc_histogram(_ptr(t), t.numel(), _ptr(counts), _stream(t)))
+        h_counts = counts.cpu()
+    return build_codebook_from_counts(h_counts, tree_format)
+
+
+def build_codebook_from_counts(counts: torch.Tensor, tree_format: int = TREE_I8):
+    """Host half of build_codebook: int64[256] counts (CPU) -> (shift, encode table, decode tree)."""
+    counts = counts.to(dtype=torch.int64, device="cpu").contiguous()
+    _require(counts.numel() == 256, "Counts tensor must have 256 elements.")
+    enc = torch.zeros(256 * 8, dtype=torch.uint8)
+    dec = torch.zeros(512 * 5, dtype=torch.uint8)
+    shift = C.c_int(0)
+    eb, db = C.c_int64(0), C.c_int64(0)
+    check(_lib.lib().kvc_build_codebook_host(C.cast(counts.data_ptr(), C.POINTER(C.c_int64)), tree_format, C.byref(shift),
+                                             _ptr(enc), enc.numel(), C.byref(eb), _ptr(dec), dec.numel(), C.byref(db)))
+    return shift.value, enc[:eb.value].clone(), dec[:db.value].clone()
+
+
+def _entropy_encode(is_k, input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
+                    base_global_offset, head_num, head_dim):
+    for t, n in ((input, "input"), (encode_code_book, "encode_code_book"), (block_infos, "block_infos"),
+                 (thread_infos, "thread_infos"), (idx_offset, "idx_offset"), (encoded_data, "encoded_data")):
+        _dev_u8(t, n)
+    tokens, stride = _geometry(input)
+    sizes = calculate_buffer_size(input, is_k, head_num, head_dim)
+    _require(block_infos.numel() >= sizes[0], "block_infos buffer too small")
+    _require(thread_infos.numel() >= sizes[1], "thread_infos buffer too small")
+    _require(idx_offset.numel() >= sizes[2], "idx_offset buffer too small")
+    total = C.c_int64(0)
+    fn = _lib.lib().kvc_k_entropy_encode if is_k else _lib.lib().kvc_v_entropy_encode
+    with torch.cuda.device(input.device):
+        check(fn(_ptr(input), tokens, stride, _ptr(encode_code_book), encode_code_book.numel(), _ptr(block_infos),
+                 _ptr(thread_infos), _ptr(idx_offset), _ptr(encoded_data), encoded_data.numel(),
+                 int(base_global_offset) & 0xFFFFFFFF, head_num, head_dim, C.byref(total), _stream(input)))
+    return encoded_data[:total.value], block_infos[:sizes[0]], thread_infos[:sizes[1]]
+
+
+def k_entropy_encode_cuda_export(input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
+                                 base_global_offset: int, head_num: int, head_dim: int):
+    """src/kernels.cu:919-966.  Returns views (payload, block_infos, thread_infos) of the caller's scratch."""
+    return _entropy_encode(True, input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
+                           base_global_offset, head_num, head_dim)
+
+
+def v_entropy_encode_cuda_export(input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
+                                 base_global_offset: int, head_num: int, head_dim: int):
+    """src/kernels.cu:968-1011."""
+    return _entropy_encode(False, input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
+                           base_global_offset, head_num, head_dim)
+
+
+def _entropy_decode(is_k, in_tensor, block_infos, thread_infos, decode_code_book, out, head_num, head_dim, tree_format):
+    for t, n in ((in_tensor, "in_tensor"), (block_infos, "block_infos"), (thread_infos, "thread_infos"),
+                 (decode_code_book, "decode_code_book"), (out, "out")):
+        _dev_u8(t, n)
+    tokens, stride = _geometry(out)
+    ms = C.c_float(0.0)
+    fn = _lib.lib().kvc_k_entropy_decode if is_k else _lib.lib().kvc_v_entropy_decode
+    with torch.cuda.device(out.device):
+        check(fn(_ptr(in_tensor), in_tensor.numel(), _ptr(block_infos), block_infos.numel(), _ptr(thread_infos),
+                 thread_infos.numel(), _ptr(decode_code_book), decode_code_book.numel(), tree_format, _ptr(out),
+                 tokens, stride, head_num, head_dim, C.byref(ms), _stream(out)))
+    return float(ms.value)
+
+
+def k_entropy_decode_cuda_export(in_tensor, block_infos, thread_infos, decode_code_book, out, head_num: int,
+                                 head_dim: int, tree_format: int = TREE_I8) -> float:
+    """src/kernels.cu:1013-1049.  Writes uint8 symbols into `out` [NB,BS,B,H,D]; returns kernel milliseconds."""
+    return _entropy_decode(True, in_tensor, block_infos, thread_infos, decode_code_book, out, head_num, head_dim, tree_format)
+
+
+def v_entropy_decode_cuda_export(in_tensor, block_infos, thread_infos, decode_code_book, out, head_num: int,
+                                 head_dim: int, tree_format: int = TREE_I8) -> float:
+    """src/kernels.cu:1051-1087."""
+    return _entropy_decode(False, in_tensor, block_infos, thread_infos, decode_code_book, out, head_num, head_dim, tree_format)
+
+
+def _fused(is_k, decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints, quant_scales, B, Cout,
+           head_num, head_dim, tree_format):
+    for t, n in ((decode_code_book, "decode_code_book"), (block_infos, "block_infos"), (thread_infos, "thread_infos"),
+                 (encoded_data, "encoded_data")):
+        _dev_u8(t, n)
+    _require(quant_min_ints.dtype == torch.int8 and quant_min_ints.is_contiguous(), "quant_min_ints must be contiguous int8")
+    _require(quant_scales.dtype == torch.float16 and quant_scales.is_contiguous(), "quant_scales must be contiguous float16")
+    _require(B.dtype == torch.float16 and B.is_contiguous() and B.dim() == 3, "B must be a contiguous 3-D float16 tensor")
+    _require(Cout.dtype == torch.float16 and Cout.is_contiguous(), "C must be a contiguous float16 tensor")
+    batch, q_heads = B.shape[0], B.shape[1]
+    if is_k:
+        _require(Cout.dim() == 3 and Cout.shape[0] == batch and Cout.shape[1] == q_heads, "C must be [batch, heads, ctx]")
+        _require(B.shape[2] == head_dim, "B must be [batch, heads, head_dim]")
+        tokens = Cout.shape[2]
+        rows = tokens // K_VEC_PER_BLK
+        n = quant_scales.numel()
+        if n == rows:
+            mask = MASK_K_BLOCK
+        elif n == rows * batch * head_num * head_dim:
+            mask = MASK_CHANNEL
+        else:
+            raise KvcompError("quant_scales has %d elements: expected one per 64-token block (%d) or one per "
+                              "(block, batch, head, channel) (%d)" % (n, rows, rows * batch * head_num * head_dim))
+    else:
+        tokens = B.shape[2]
+        _require(Cout.dim() == 4 and Cout.shape[0] * V_VEC_LEN == tokens and Cout.shape[1] == batch
+                 and Cout.shape[2] == q_heads and Cout.shape[3] == head_dim, "C must be [ctx/128, batch, heads, head_dim]")
+        n = quant_scales.numel()
+        if n == tokens:
+            mask = MASK_V_TOKEN
+        elif n == tokens * batch:
+            mask = MASK_SIM_TOKEN
+        elif n == tokens * batch * head_num:
+            mask = MASK_VECTOR
+        else:
+            raise KvcompError("quant_scales has %d elements: expected one per token (%d), per (token, batch) or per "
+                              "(token, batch, head)" % (n, tokens))
+    _require(quant_min_ints.numel() == n, "quant_min_ints and quant_scales must have the same number of elements")
+    ms = C.c_float(0.0)
+    fn = _lib.lib().kvc_k_decode_and_mat_vec_mul if is_k else _lib.lib().kvc_v_decode_and_mat_vec_mul
+    with torch.cuda.device(B.device):
+        check(fn(_ptr(decode_code_book), decode_code_book.numel(), tree_format, _ptr(block_infos), block_infos.numel(),
+                 _ptr(thread_infos), thread_infos.numel(), _ptr(encoded_data), encoded_data.numel(),
+                 _ptr(quant_min_ints), _ptr(quant_scales), mask, _ptr(B), _ptr(Cout), tokens, batch, head_num, q_heads,
+                 head_dim, C.byref(ms), _stream(B)))
+    return float(ms.value)
+
+
+def k_decode_and_mat_vec_mul_cuda_export(decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints,
+                                         quant_scales, B, C, head_num: int, head_dim: int,
+                                         tree_format: int = TREE_I8) -> float:
+    """src/kernels.cu:1093-1136.  C[b,h,t] = sum_i dequant(K)[t,b,h,i] * B[b,h,i]; returns kernel milliseconds."""
+    return _fused(True, decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints, quant_scales, B, C,
+                  head_num, head_dim, tree_format)
+
+
+def v_decode_and_mat_vec_mul_cuda_export(decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints,
+                                         quant_scales, B, C, head_num: int, head_dim: int,
+                                         tree_format: int = TREE_I8) -> float:
+    """src/kernels.cu:1138-1180.  C[g,b,h,d] = sum_{t<128} dequant(V)[128g+t,b,h,d] * B[b,h,128g+t]."""
+    return _fused(False, decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints, quant_scales, B, C,
+                  head_num, head_dim, tree_format)
+
+
+def k_mat_vec_mul_cuda_export(k: torch.Tensor, q: torch.Tensor, out: torch.Tensor) -> float:
+    """src/kernels.cu:1221-1273: dense fp16 baseline, out[t,b,h] = sum_i k[t,b,h,i] * q[b,h,i]."""
+    _require(k.dim() == 4 and q.dim() == 3 and out.dim() == 3, "k [ctx,B,H,D], q [B,H,D], out [ctx,B,H]")
+    ctx, batch, heads, dim = k.shape
+    _require(q.shape[0] == batch, "Batch size of A and B must be equal")
+    _require(q.shape[1] == heads, "Head num of A and B must be equal")
+    _require(q.shape[2] == dim, "Head dim of A and B must be equal")
+    _require(tuple(out.shape) == (ctx, batch, heads), "out must be [ctx, batch, heads]")
+    for t, n in ((k, "A"), (q, "B"), (out, "C")):
+        _require(t.dtype == torch.float16, "%s must be of type half" % n)
+        _require(t.is_contiguous(), "%s must be contiguous" % n)
+    ms = C.c_float(0.0)
+    with torch.cuda.device(k.device):
+        check(_lib.lib().kvc_k_mat_vec_mul(_ptr(k), _ptr(q), _ptr(out), ctx, batch, heads, dim, C.byref(ms), _stream(k)))
+    return float(ms.value)
