@@ -139,6 +139,30 @@ int kvc_v_decode_and_mat_vec_mul(const uint8_t *d_decode_tree, int64_t decode_tr
                                  int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                                  float *elapsed_ms, void *stream);
 
+/* ---- decode tables built once (no counterpart in the reference, which walks its tree bit by bit) ----
+ * The decoders look symbols up in a table derived from the decode tree.  The reference-signature entry
+ * points above derive it on every call; these take tables prepared once per codebook:
+ *   kvc_build_lut: n_codebooks trees, tree_stride_bytes apart, each tree_bytes long -> d_luts
+ *                  (n_codebooks * kvc_lut_bytes() bytes, 16-byte aligned).
+ *   kvc_k_scores_lut / kvc_v_partials_lut: as kvc_k_/v_decode_and_mat_vec_mul, plus
+ *     rows_per_codebook: tile rows (64 tokens for K, 128 for V) that share one table; 0 = one table for all
+ *     out_f32:           1 writes fp32 results instead of fp16. */
+int64_t kvc_lut_bytes(void);
+int kvc_build_lut(const uint8_t *d_decode_trees, int64_t tree_bytes, int tree_format, int64_t n_codebooks,
+                  int64_t tree_stride_bytes, void *d_luts, void *stream);
+int kvc_k_scores_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
+                     int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                     const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
+                     const void *d_quant_scales_f16, int quant_mask, const void *d_q_f16, void *d_scores,
+                     int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
+                     int64_t head_dim, float *elapsed_ms, void *stream);
+int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
+                       int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                       const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
+                       const void *d_quant_scales_f16, int quant_mask, const void *d_p_f16, void *d_partial,
+                       int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
+                       int64_t head_dim, float *elapsed_ms, void *stream);
+
 /* ---- dense baseline: k_mat_vec_mul_cuda_export (kernels.cu:1182-1273) ------------------------------
  * d_k fp16 [tokens, batch, heads, head_dim], d_q fp16 [batch, heads, head_dim],
  * d_out fp16 [tokens, batch, heads].  (The reference requires batch == 1 and head_dim == 128.) */

@@ -26,12 +26,18 @@ _SIGNATURES = {
                                      _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,
                                      _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_lut_bytes": [],
+    "kvc_build_lut": [_vp, _i64, _int, _i64, _i64, _vp, _vp],
+    "kvc_k_scores_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int,
+                         _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_v_partials_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int,
+                           _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_k_mat_vec_mul": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_quant_groups": [_i64, _i64, _i64, _i64, _i64, _int],
     "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }
-_RESTYPES = {"kvc_quant_groups": _i64}
+_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64}
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["kvc_last_error"])
 

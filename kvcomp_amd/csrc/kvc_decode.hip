@@ -373,7 +373,8 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                      int64_t thread_infos_bytes, const uint8_t *d_encoded, int64_t encoded_bytes,
                      const int8_t *d_min, const void *d_scale, int quant_mask, const void *d_x, void *d_out,
                      int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
-                     float *elapsed_ms, void *stream_)
+                     float *elapsed_ms, void *stream_, const uint32_t *d_luts = nullptr, int rows_per_codebook = 0,
+                     int out_f32 = 0)
 {
     hipStream_t stream = (hipStream_t)stream_;
     if (tokens == 0) {
@@ -391,27 +392,33 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                     "fused V supports per-token quantization groups (0xE, 0xC, 0x8)");
         KVC_REQUIRE(head_dim % KVC_WAVE == 0, "fused V needs head_dim to be a multiple of 64");
     }
-    void *slot;
-    if (int rc = kvc_workspace_slot(&slot)) return rc;
+    void *slot = nullptr;
+    if (!d_luts) {
+        if (int rc = kvc_workspace_slot(&slot)) return rc;
+    }
     KvcFusedArgs a;
     int64_t rows;
     const int64_t stride = batch * kv_heads * head_dim;
     if (int rc = kvc_fill_stream_args(a.s, d_encoded, encoded_bytes, d_block_infos, block_infos_bytes, d_thread_infos,
-                                      thread_infos_bytes, (const uint32_t *)slot, is_k, tokens, stride, head_dim, &rows))
+                                      thread_infos_bytes, d_luts ? d_luts : (const uint32_t *)slot, is_k, tokens, stride,
+                                      head_dim, &rows))
         return rc;
+    a.s.rows_per_codebook = d_luts ? rows_per_codebook : 0;
     a.min_i8 = d_min;
     a.scale = reinterpret_cast<const __half *>(d_scale);
     a.quant_mask = quant_mask;
     a.x = reinterpret_cast<const __half *>(d_x);
     a.out = d_out;
-    a.out_f32 = 0;
+    a.out_f32 = out_f32;
     a.tokens = tokens;
     a.batch = (int)batch;
     a.kv_heads = (int)kv_heads;
     a.q_heads = (int)q_heads;
     a.head_dim = (int)head_dim;
     KvcTimer timer(elapsed_ms, stream);
-    if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
+    if (!d_luts) {
+        if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
+    }
     const dim3 grid = kvc_grid(a.s, rows);
     switch (rep) {
         case 1: kvc_launch_fused<1>(is_k, a, grid, stream); break;
@@ -449,4 +456,46 @@ extern "C" int kvc_v_decode_and_mat_vec_mul(const uint8_t *d_decode_tree, int64_
     return kvc_fused(0, d_decode_tree, decode_tree_bytes, tree_format, d_block_infos, block_infos_bytes, d_thread_infos,
                      thread_infos_bytes, d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask,
                      d_p_f16, d_partial_f16, tokens, batch, kv_heads, q_heads, head_dim, elapsed_ms, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// variants that take decode tables built once with kvc_build_lut (no per-call table construction)
+// ---------------------------------------------------------------------------------------------------
+extern "C" int64_t kvc_lut_bytes(void) { return KVC_LUT_BYTES; }
+
+extern "C" int kvc_build_lut(const uint8_t *d_decode_trees, int64_t tree_bytes, int tree_format, int64_t n_codebooks,
+                             int64_t tree_stride_bytes, void *d_luts, void *stream)
+{
+    KVC_REQUIRE(n_codebooks >= 1 && n_codebooks <= 65535, "bad codebook count");
+    KVC_REQUIRE(((uintptr_t)d_luts & 15) == 0, "table buffer must be 16-byte aligned");
+    return kvc_launch_build_lut(d_decode_trees, tree_bytes, tree_format, (uint32_t *)d_luts, (int)n_codebooks,
+                                tree_stride_bytes, (hipStream_t)stream);
+}
+
+extern "C" int kvc_k_scores_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
+                                int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                                const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
+                                const void *d_quant_scales_f16, int quant_mask, const void *d_q_f16, void *d_scores,
+                                int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
+                                int64_t head_dim, float *elapsed_ms, void *stream)
+{
+    KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
+    return kvc_fused(1, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
+                     d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_q_f16, d_scores, tokens,
+                     batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
+                     (int)rows_per_codebook, out_f32);
+}
+
+extern "C" int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
+                                  int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                                  const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
+                                  const void *d_quant_scales_f16, int quant_mask, const void *d_p_f16, void *d_partial,
+                                  int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
+                                  int64_t head_dim, float *elapsed_ms, void *stream)
+{
+    KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
+    return kvc_fused(0, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
+                     d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_p_f16, d_partial, tokens,
+                     batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
+                     (int)rows_per_codebook, out_f32);
 }

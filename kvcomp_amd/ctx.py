@@ -1,0 +1,320 @@
+"""Compressed KV-cache context: the object layout and methods of the reference's KVCompCtx
+(models/cache/kvcomp_encode.py:15-326), with every device step running through libkvcomp_hip.
+
+Same attribute names (encoded_data, block_infos, thread_infos, quant_min_ints, quant_scales, encode_codebook,
+decode_codebook, buffer, ctx_len, compressed_ctx_len, shape) and the same method contracts (store, get,
+get_only_compressed, get_decode_quant_ints, mat_vec_mul, build_codebook, get_cr).  Differences:
+
+  * the quantizer is one HIP launch instead of ~8 fp16 PyTorch kernels (bit-identical symbols);
+  * encoder scratch is kept per device and only grows (the reference re-allocates and zero-fills four
+    buffers on every store, kvcomp_encode.py:88-95), and the accumulated stream lives in amortised
+    growable buffers instead of being re-concatenated on every store (kvcomp_encode.py:129-133);
+  * batch > 1 and per-channel K (QuantMode.ChannelQuant) are accepted.
+"""
+import ast
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from . import kvcomp_cuda
+from .compute import QUANT_MODE_MAP, QuantMode, cut_tensor_ctx_len_0, dequant, quant, safe_cat  # noqa: F401
+
+
+class ExtractCacheConfig:
+    """utils/config.py:3-19"""
+
+    def __init__(self, collect_round: int):
+        self.collect_round = collect_round
+        self.key_caches = {}
+        self.value_caches = {}
+
+    def size(self):
+        total = 0
+        for caches in (self.key_caches, self.value_caches):
+            for per_round in caches.values():
+                for t in per_round.values():
+                    total += t.numel() * 16
+        return total
+
+
+class KVCompCacheConfig:
+    """utils/config.py:21-140: the eleven configuration fields, printable and parseable."""
+
+    _FIELDS = ("enable_quant", "model_name", "enable_pre_rope", "k_quant_mode", "v_quant_mode", "k_block_size",
+               "v_block_size", "k_recent_size", "v_recent_size", "k_quant_scale_rel", "v_quant_scale_rel")
+
+    def __init__(self, model_name, k_quant_mode, v_quant_mode, k_block_size, v_block_size, k_recent_size,
+                 v_recent_size, k_quant_scale_rel, v_quant_scale_rel, enable_quant=True, enable_pre_rope=False):
+        self.enable_quant = enable_quant
+        self.model_name = model_name
+        self.enable_pre_rope = enable_pre_rope
+        self.k_quant_mode = k_quant_mode
+        self.v_quant_mode = v_quant_mode
+        self.k_block_size = k_block_size
+        self.v_block_size = v_block_size
+        self.k_recent_size = k_recent_size
+        self.v_recent_size = v_recent_size
+        self.k_quant_scale_rel = k_quant_scale_rel
+        self.v_quant_scale_rel = v_quant_scale_rel
+
+    def __str__(self):
+        d = {"enable_quant": self.enable_quant, "enable_pre_rope": self.enable_pre_rope, "model_name": self.model_name}
+        if self.enable_quant:
+            d.update(k_quant_mode=self.k_quant_mode.value, v_quant_mode=self.v_quant_mode.value,
+                     k_block_size=self.k_block_size, v_block_size=self.v_block_size,
+                     k_recent_size=self.k_recent_size, v_recent_size=self.v_recent_size,
+                     k_quant_scale_rel=self.k_quant_scale_rel, v_quant_scale_rel=self.v_quant_scale_rel)
+        return str(d)
+
+    __repr__ = __str__
+
+    @staticmethod
+    def from_str(text: str):
+        d = ast.literal_eval(text)       # the reference uses eval (utils/config.py:71); literals are all it needs
+        if d["enable_quant"]:
+            kw = dict(k_quant_mode=QuantMode(d["k_quant_mode"]), v_quant_mode=QuantMode(d["v_quant_mode"]),
+                      k_block_size=d["k_block_size"], v_block_size=d["v_block_size"],
+                      k_recent_size=d["k_recent_size"], v_recent_size=d["v_recent_size"],
+                      k_quant_scale_rel=d["k_quant_scale_rel"], v_quant_scale_rel=d["v_quant_scale_rel"])
+        else:
+            kw = dict(k_quant_mode=None, v_quant_mode=None, k_block_size=None, v_block_size=None, k_recent_size=None,
+                      v_recent_size=None, k_quant_scale_rel=None, v_quant_scale_rel=None)
+        return KVCompCacheConfig(model_name=d["model_name"], enable_quant=d["enable_quant"],
+                                 enable_pre_rope=d["enable_pre_rope"], **kw)
+
+    def _key(self):
+        return tuple(getattr(self, f) for f in self._FIELDS)
+
+    def __eq__(self, other):
+        return isinstance(other, KVCompCacheConfig) and self._key() == other._key()
+
+    def __hash__(self):
+        return hash(self._key())
+
+
+class KVCompCacheConfigStatic:
+    """Process-wide configuration slot (models/cache/kvcomp_quant.py:10-12)."""
+    config: Optional[KVCompCacheConfig] = None
+    extract_cache: Optional[ExtractCacheConfig] = None
+
+
+class _Growable:
+    """Device buffer that grows geometrically along dim 0; `.view` is the filled prefix."""
+
+    def __init__(self):
+        self.data: Optional[torch.Tensor] = None
+        self.used = 0
+
+    def append(self, t: torch.Tensor):
+        n = t.shape[0]
+        if self.data is None:
+            cap = max(2 * n, 1)
+            self.data = torch.empty((cap,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+        elif self.used + n > self.data.shape[0]:
+            cap = max(2 * self.data.shape[0], self.used + n)
+            grown = torch.empty((cap,) + tuple(self.data.shape[1:]), dtype=self.data.dtype, device=self.data.device)
+            grown[:self.used] = self.data[:self.used]
+            self.data = grown
+        self.data[self.used:self.used + n] = t
+        self.used += n
+
+    @property
+    def view(self) -> Optional[torch.Tensor]:
+        return None if self.data is None else self.data[:self.used]
+
+
+class KVCompCtx:
+    """One compressed K or V stream of one layer (models/cache/kvcomp_encode.py:15-326)."""
+
+    # encoder scratch shared by every context on a device (kvcomp_encode.py:17-21); grown, never shrunk
+    buffer_ctx_len: Dict[torch.device, int] = dict()
+    block_infos_buffer: Dict[torch.device, torch.Tensor] = dict()
+    thread_infos_buffer: Dict[torch.device, torch.Tensor] = dict()
+    idx_offset_buffer: Dict[torch.device, torch.Tensor] = dict()
+    pre_alloc_compressed_data_buffer: Dict[torch.device, torch.Tensor] = dict()
+
+    def __init__(self, is_k: bool, batch_size: int, head_num: int, head_dim: int, quant_scale_rel: float,
+                 encode_codebook_path: str = None, decode_codebook_path: str = None):
+        cfg = KVCompCacheConfigStatic.config
+        assert cfg is not None, "KVCompCacheConfigStatic.config is None"
+        assert cfg.k_quant_mode in (QuantMode.BlockQuant, QuantMode.ChannelQuant), \
+            "k_quant_mode must be BlockQuant or ChannelQuant for the kernel implementation"
+        assert cfg.v_quant_mode in (QuantMode.TokenQuant, QuantMode.VectorQuant), \
+            "v_quant_mode must be TokenQuant or VectorQuant for the kernel implementation"
+        assert head_dim <= kvcomp_cuda.K_VEC_LEN and head_dim % 8 == 0, "head_dim must be a multiple of 8, at most K_VEC_LEN"
+        self.is_k = is_k
+        self.batch_size = batch_size
+        self.head_num = head_num
+        self.head_dim = head_dim
+        self.quant_scale_rel = quant_scale_rel
+        self.ctx_len = 0
+        self.compressed_ctx_len = 0
+        self.device: Optional[torch.device] = None
+        self.quant_dims = QUANT_MODE_MAP[cfg.k_quant_mode] if is_k else QUANT_MODE_MAP[cfg.v_quant_mode]
+        self.block_size = cfg.k_block_size if is_k else cfg.v_block_size
+        self.recent_size = cfg.k_recent_size if is_k else cfg.v_recent_size
+        if is_k:
+            assert (batch_size * head_num * head_dim) % head_dim == 0
+            assert self.block_size == kvcomp_cuda.K_VEC_PER_BLK, "for K, block size must equal VEC_PER_BLK"
+        else:
+            assert (batch_size * head_num * head_dim) % kvcomp_cuda.V_VEC_PER_BLK == 0, "hidden size must be divisible by VEC_PER_BLK"
+            assert self.block_size % kvcomp_cuda.V_VEC_LEN == 0, "block size must be divisible by VEC_LEN"
+        self._encoded = _Growable()
+        self._block_infos = _Growable()
+        self._thread_infos = _Growable()
+        self._min_ints = _Growable()
+        self._scales = _Growable()
+        self.buffer: Optional[torch.Tensor] = None
+        self.encode_codebook: Optional[torch.Tensor] = None
+        self.decode_codebook: Optional[torch.Tensor] = None
+
+    # the reference's public tensor attributes (kvcomp_encode.py:56-61)
+    encoded_data = property(lambda self: self._encoded.view)
+    block_infos = property(lambda self: self._block_infos.view)
+    thread_infos = property(lambda self: self._thread_infos.view)
+    quant_min_ints = property(lambda self: self._min_ints.view)
+    quant_scales = property(lambda self: self._scales.view)
+
+    def _check(self, cache: torch.Tensor):
+        assert cache.dtype == torch.float16, "cache must be float16"
+        assert cache.shape[1] == self.batch_size, "batch size mismatch"
+        assert cache.shape[2] == self.head_num, "head num mismatch"
+        assert cache.shape[3] == self.head_dim, "head dim mismatch"
+
+    def _scratch(self, sizes):
+        dev = self.device
+        for store, n in ((KVCompCtx.block_infos_buffer, sizes[0]), (KVCompCtx.thread_infos_buffer, sizes[1]),
+                         (KVCompCtx.idx_offset_buffer, sizes[2]), (KVCompCtx.pre_alloc_compressed_data_buffer, sizes[3])):
+            if dev not in store or store[dev].numel() < n:
+                store[dev] = torch.empty(n, dtype=torch.uint8, device=dev)
+        return (KVCompCtx.block_infos_buffer[dev], KVCompCtx.thread_infos_buffer[dev],
+                KVCompCtx.idx_offset_buffer[dev], KVCompCtx.pre_alloc_compressed_data_buffer[dev])
+
+    def store(self, cache: torch.Tensor):
+        """kvcomp_encode.py:69-136: append [T_new, B, H, D]; compress the whole blocks that leave the tail.
+        Returns the uint8 symbols that were compressed (None if nothing left the tail)."""
+        self._check(cache)
+        if self.device is None:
+            self.device = cache.device
+        assert self.device == cache.device, "device mismatch"
+        self.ctx_len += cache.shape[0]
+        to_compress, self.buffer = cut_tensor_ctx_len_0(self.buffer, cache, self.block_size, self.recent_size, dim=0)
+        if to_compress is None:
+            return None
+        blocked = to_compress.reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
+        quant_ints, min_ints, quant_scale = quant(blocked, self.quant_dims, self.quant_scale_rel)
+        sizes = kvcomp_cuda.calculate_buffer_size(quant_ints, self.is_k, self.head_num, self.head_dim)
+        KVCompCtx.buffer_ctx_len[self.device] = to_compress.shape[0]
+        bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
+        if self.encode_codebook is None:     # first stored chunk defines the codebook (kvcomp_encode.py:99-103)
+            shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
+            assert shift == 0, "shift must be 0"
+            self.encode_codebook = enc.to(self.device)
+            self.decode_codebook = dec.to(self.device)
+        fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
+        encoded_, block_infos_, vec_infos_ = fn(quant_ints, self.encode_codebook, bi_buf, ti_buf, idx_buf, payload_buf,
+                                                self._encoded.used, self.head_num, self.head_dim)
+        self._encoded.append(encoded_)
+        self._block_infos.append(block_infos_)
+        self._thread_infos.append(vec_infos_)
+        self._min_ints.append(min_ints)
+        self._scales.append(quant_scale)
+        self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
+        return quant_ints
+
+    def _assert_ready(self):
+        assert self.quant_min_ints is not None, "quant_min_ints is None"
+        assert self.quant_scales is not None, "quant_scales is None"
+        assert self.encoded_data is not None, "encoded_data is None"
+        assert self.block_infos is not None, "huffman_block_info is None"
+        assert self.thread_infos is not None, "huffman_thread_info is None"
+        assert self.decode_codebook is not None, "decode_codebook is None"
+
+    def get_decode_quant_ints(self) -> Tuple[torch.Tensor, float]:
+        """kvcomp_encode.py:168-207: Huffman-decode the whole compressed part back to uint8 symbols."""
+        self._assert_ready()
+        decoded = torch.empty(self.compressed_ctx_len // self.block_size, self.block_size, self.batch_size,
+                              self.head_num, self.head_dim, dtype=torch.uint8, device=self.device)
+        fn = kvcomp_cuda.k_entropy_decode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_decode_cuda_export
+        t_ms = fn(self.encoded_data, self.block_infos, self.thread_infos, self.decode_codebook, decoded,
+                  self.head_num, self.head_dim)
+        return decoded, t_ms
+
+    def get_only_compressed(self) -> Tuple[torch.Tensor, float]:
+        """kvcomp_encode.py:153-166: decode + dequantize the compressed part -> ([ctx_c, B, H, D] fp16, ms)."""
+        decoded, t_ms = self.get_decode_quant_ints()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        out = dequant(decoded, self.quant_min_ints, self.quant_scales, self.quant_dims)
+        end.record()
+        end.synchronize()
+        return out.flatten(0, 1), t_ms + start.elapsed_time(end)
+
+    def get(self) -> Tuple[torch.Tensor, float]:
+        """kvcomp_encode.py:138-151: compressed part followed by the uncompressed tail."""
+        out, t_ms = self.get_only_compressed()
+        if self.buffer is not None and self.buffer.shape[0] > 0:
+            out = torch.cat([out, self.buffer], dim=0)
+        return out, t_ms
+
+    def mat_vec_mul(self, B: torch.Tensor) -> Tuple[torch.Tensor, float]:
+        """kvcomp_encode.py:209-280.  K: B = q [B, H, D] -> scores [B, H, ctx_c].  V: B = p [B, H, ctx_c] ->
+        [1, B, H, D] (the per-128-token partials summed, as the reference does in PyTorch)."""
+        self._assert_ready()
+        assert B.dtype == torch.float16, "B must be float16"
+        assert len(B.shape) == 3, "B must be 3D tensor"
+        assert B.shape[0] == self.batch_size, "batch size mismatch"
+        assert B.shape[1] % self.head_num == 0, "head num mismatch"
+        q_heads = B.shape[1]
+        if self.is_k:
+            assert B.shape[2] == self.head_dim, "head dim mismatch"
+            C = torch.empty(self.batch_size, q_heads, self.compressed_ctx_len, dtype=torch.float16, device=self.device)
+            t_ms = kvcomp_cuda.k_decode_and_mat_vec_mul_cuda_export(
+                self.decode_codebook, self.block_infos, self.thread_infos, self.encoded_data,
+                self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim)
+            return C, t_ms
+        assert B.shape[2] == self.compressed_ctx_len, "ctx len mismatch"
+        C = torch.empty(self.compressed_ctx_len // kvcomp_cuda.V_VEC_LEN, self.batch_size, q_heads, self.head_dim,
+                        dtype=torch.float16, device=self.device)
+        t_ms = kvcomp_cuda.v_decode_and_mat_vec_mul_cuda_export(
+            self.decode_codebook, self.block_infos, self.thread_infos, self.encoded_data,
+            self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        C = C.sum(dim=0, keepdim=True, dtype=torch.float32).to(torch.float16)
+        end.record()
+        end.synchronize()
+        return C, t_ms + start.elapsed_time(end)
+
+    def build_codebook(self, tensors: List[torch.Tensor]):
+        """kvcomp_encode.py:282-306: one codebook from the quantized whole blocks of sample tensors."""
+        assert len(tensors) > 0, "tensors must not be empty"
+        device_ = tensors[0].device
+        sym = []
+        for cache in tensors:
+            self._check(cache)
+            assert device_ == cache.device, "device mismatch"
+            blocked_len = cache.shape[0] // self.block_size * self.block_size
+            blocked = cache[:blocked_len].reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
+            sym.append(quant(blocked, self.quant_dims, self.quant_scale_rel)[0])
+        shift, enc, dec = kvcomp_cuda.build_codebook(sym)
+        assert shift == 0, "shift must be 0"
+        if self.device is None:
+            self.device = device_
+            KVCompCtx.buffer_ctx_len[self.device] = 0
+        self.encode_codebook = enc.to(self.device)
+        self.decode_codebook = dec.to(self.device)
+
+    @property
+    def shape(self):
+        return torch.Size([self.compressed_ctx_len, self.batch_size, self.head_num, self.head_dim])
+
+    def compressed_bytes(self) -> int:
+        """Denominator of get_cr (kvcomp_encode.py:318-324): everything a fused kernel has to read."""
+        return (self.block_infos.numel() + self.thread_infos.numel() + self.encoded_data.numel() +
+                self.quant_min_ints.numel() + self.quant_scales.numel() * 2)
+
+    def get_cr(self):
+        """kvcomp_encode.py:317-326"""
+        original = 2 * self.batch_size * self.compressed_ctx_len * self.head_num * self.head_dim
+        return original / self.compressed_bytes()

@@ -1,0 +1,164 @@
+"""GPU tests of the compressed-cache context, modelled on the reference's own scripts: exact symbol round
+trip after two appended stores (kvcomp_cuda_extension/scripts/test_py_ctx_k_2d_load.py:55-84, test_py_ctx_v.py),
+repeated get (scripts/test_py_ctx_multiple_get.py:22-30), fused result against a dense matmul on the
+dequantized cache (test_py_ctx_k_2d_load.py:129-134, here at 1e-3 instead of 1e-2), and prefill-then-append-one
+(accuracy/reproduce_cuda_error.py:25-46)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as O
+from tests import _synth as S
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _config(k_mode="BlockQuant", v_mode="TokenQuant", k_recent=64, v_recent=128, ebk=0.1, ebv=0.2):
+    from kvcomp_amd.ctx import KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("synthetic", QuantMode(k_mode), QuantMode(v_mode), 64, 128,
+                                                       k_recent, v_recent, ebk, ebv)
+
+
+def _oracle_mask(ctx):
+    from kvcomp_amd.compute import dims_to_mask
+    return dims_to_mask(ctx.quant_dims)
+
+
+@pytest.mark.parametrize("is_k,mode", [(True, "BlockQuant"), (True, "ChannelQuant"), (False, "TokenQuant"), (False, "VectorQuant")])
+def test_twice_store_round_trip_and_get(is_k, mode):
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode=mode if is_k else "BlockQuant", v_mode=mode if not is_k else "TokenQuant")
+    T, B, H, D = 1024, 1, 8, 128
+    x = (S.synth_k if is_k else S.synth_v)(T, B, H, D)
+    eb = 0.03 if is_k else 0.07                     # the reference scripts' error bounds
+    ctx = KVCompCtx(is_k, B, H, D, eb)
+    ctx.build_codebook([x.to(DEV), x.to(DEV)])
+    q1 = ctx.store(x.to(DEV))
+    q2 = ctx.store(x.to(DEV))
+    assert ctx.ctx_len == 2 * T and ctx.compressed_ctx_len == 2 * T and ctx.buffer.shape[0] == 0
+    quant_int = torch.cat([q1, q2], dim=0)
+    decoded, ms = ctx.get_decode_quant_ints()
+    assert torch.equal(decoded, quant_int)
+    # symbols, min and scale equal the oracle's, store by store
+    mask = _oracle_mask(ctx)
+    o = O.quant(S.np16(S.blocked(x, ctx.block_size)), mask, eb)
+    assert np.array_equal(q1.cpu().numpy(), o[3]) and np.array_equal(q2.cpu().numpy(), o[3])
+    n = ctx.quant_scales.shape[0] // 2
+    assert np.array_equal(ctx.quant_scales[:n].cpu().numpy().view(np.uint16), o[2].view(np.uint16))
+    assert np.array_equal(ctx.quant_min_ints[n:].cpu().numpy(), o[4])
+    # per-tile stream equals the oracle's encoder run with this context's codebook (second store: base offset)
+    p1, bi1, ti1 = O.encode_tiles(o[3], is_k, ctx.encode_codebook.cpu().numpy(), 0)
+    p2, bi2, ti2 = O.encode_tiles(o[3], is_k, ctx.encode_codebook.cpu().numpy(), p1.size)
+    assert np.array_equal(ctx.encoded_data.cpu().numpy(), np.concatenate([p1, p2]))
+    assert np.array_equal(ctx.block_infos.cpu().numpy(), np.concatenate([bi1, bi2]))
+    assert np.array_equal(ctx.thread_infos.cpu().numpy(), np.concatenate([ti1, ti2]))
+    # get(): bit-exact dequantized cache, idempotent
+    full, _ = ctx.get()
+    deq = O.dequant(o[3], o[4], o[2], mask).reshape(T, B, H, D)
+    assert np.array_equal(full[:T].cpu().numpy().view(np.uint16), deq.view(np.uint16))
+    assert np.array_equal(full[T:].cpu().numpy().view(np.uint16), deq.view(np.uint16))
+    again, _ = ctx.get()
+    assert torch.equal(full, again)
+    # compression ratio formula (models/cache/kvcomp_encode.py:317-326)
+    comp = (ctx.block_infos.numel() + ctx.thread_infos.numel() + ctx.encoded_data.numel() +
+            ctx.quant_min_ints.numel() + 2 * ctx.quant_scales.numel())
+    assert ctx.get_cr() == pytest.approx(2 * B * 2 * T * H * D / comp)
+    assert tuple(ctx.shape) == (2 * T, B, H, D)
+
+
+@pytest.mark.parametrize("is_k,mode", [(True, "BlockQuant"), (True, "ChannelQuant"), (False, "TokenQuant")])
+def test_fused_mat_vec_mul_against_dense(is_k, mode):
+    from kvcomp_amd.ctx import KVCompCtx
+    import kvcomp_amd.kvcomp_cuda as m
+    _config(k_mode=mode if is_k else "BlockQuant")
+    T, B, H, D = 2048, 1, 8, 128
+    x = (S.synth_k if is_k else S.synth_v)(T, B, H, D).to(DEV)
+    ctx = KVCompCtx(is_k, B, H, D, 0.1 if is_k else 0.2)
+    ctx.store(x)
+    dense, _ = ctx.get_only_compressed()
+    if is_k:
+        q = S.synth_q(B, H, D).to(DEV)
+        C, ms = ctx.mat_vec_mul(q)
+        ref = torch.einsum("tbhd,bhd->bht", dense.float(), q.float())
+        assert (C.float() - ref).abs().max() <= 1e-3 * ref.abs().max()
+        base = torch.empty(T, B, H, dtype=torch.float16, device=DEV)
+        m.k_mat_vec_mul_cuda_export(dense.contiguous(), q, base)         # the dense baseline on the same cache
+        assert (base.float().permute(1, 2, 0) - ref).abs().max() <= 1e-3 * ref.abs().max()
+    else:
+        p = S.synth_p(B, H, T).to(DEV)
+        C, ms = ctx.mat_vec_mul(p)
+        ref = torch.einsum("tbhd,bht->bhd", dense.float(), p.float())
+        assert tuple(C.shape) == (1, B, H, D)
+        assert (C.float()[0] - ref).abs().max() <= 1e-3 * ref.abs().max()
+    assert ms > 0
+
+
+def test_prefill_then_append_one_token_at_a_time():
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(v_recent=256)
+    T0, extra, B, H, D = 952, 300, 1, 4, 128
+    x = S.synth_v(T0 + extra, B, H, D).to(DEV)
+    ctx = KVCompCtx(False, B, H, D, 0.04)
+    ctx.store(x[:T0].contiguous())
+    for i in range(T0, T0 + extra):
+        ctx.store(x[i:i + 1].contiguous())
+        if i % 50 == 0:
+            full, _ = ctx.get()
+            assert full.shape[0] == i + 1
+    full, _ = ctx.get()
+    assert ctx.ctx_len == T0 + extra and full.shape[0] == T0 + extra
+    c = ctx.compressed_ctx_len
+    assert c % 128 == 0 and 128 <= ctx.ctx_len - c < 256 + 128 and ctx.buffer.shape[0] == ctx.ctx_len - c
+    assert torch.equal(full[c:], x[c:])                                # the tail is stored verbatim
+    # the compressed part: per-token quantization does not depend on how the tokens were chunked
+    o = O.quant(S.np16(S.blocked(x[:c].cpu(), 128)), O.MASK_V_TOKEN, 0.04)
+    deq = O.dequant(o[3], o[4], o[2], O.MASK_V_TOKEN).reshape(c, B, H, D)
+    assert np.array_equal(full[:c].cpu().numpy().view(np.uint16), deq.view(np.uint16))
+    assert np.array_equal(ctx.get_decode_quant_ints()[0].cpu().numpy(), o[3])
+
+
+def test_batch_and_gqa_heads():
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant")
+    T, B, H, D, rep = 512, 2, 2, 128, 4
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    s, _ = kctx.mat_vec_mul(q)
+    kd, _ = kctx.get_only_compressed()
+    ref = torch.einsum("tbhd,bhd->bht", kd.float().repeat_interleave(rep, dim=2), q.float())
+    assert (s.float() - ref).abs().max() <= 1e-3 * ref.abs().max()
+    p = torch.softmax(s.float() / D ** 0.5, dim=-1).half()
+    o, _ = vctx.mat_vec_mul(p)
+    vd, _ = vctx.get_only_compressed()
+    ref = torch.einsum("tbhd,bht->bhd", vd.float().repeat_interleave(rep, dim=2), p.float())
+    assert (o.float()[0] - ref).abs().max() <= 1e-3 * ref.abs().max()
+
+
+def test_smoke_entry():
+    import __graft_entry__ as g
+    g.smoke()
+
+
+@pytest.mark.parametrize("k_mode,rep,extra", [("ChannelQuant", 1, 0), ("ChannelQuant", 4, 37), ("BlockQuant", 2, 200)])
+def test_compressed_attention_matches_fp32_reference(k_mode, rep, extra):
+    """Full decode attention (scores -> 1/sqrt(d) -> softmax -> p.V, grouped-query heads, uncompressed tails)
+    against fp32 PyTorch attention over the dequantized cache: 1e-3 relative to max|out|."""
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode=k_mode)
+    T, B, H, D = 1024 + extra, 2, 2, 128
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    out = CompressedAttention(kctx, vctx).attend(q)
+    kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+    assert kd.shape[0] == T and vd.shape[0] == T
+    s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
+    ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
+    assert (out - ref).abs().max() <= 1e-3 * ref.abs().max()

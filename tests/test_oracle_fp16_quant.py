@@ -103,12 +103,12 @@ def test_quant_closed_form_small_case():
     s16, m16, c16, s8, m8 = O.quant(x, O.MASK_K_BLOCK, 0.1)
     assert float(c16.ravel()[0]) == 0.5 and int(m8.ravel()[0]) == 0
     assert s8.reshape(-1)[:xs.size].tolist() == [0, 0, 1, 2, 2, 2, 5, 9, 10]     # 0.5 -> 0 and 2.5 -> 2: ties to even
-    # shifting every value by -1.5 (= -3 steps) moves min_i to -3 and leaves the symbols alone
-    s16b, m16b, c16b, s8b, m8b = O.quant((x.astype(np.float32) - 1.5).astype(np.float16), O.MASK_K_BLOCK, 0.1)
-    assert int(m8b.ravel()[0]) == -3 and np.array_equal(s8b, s8)
+    # shifting every value by -2 (= -4 steps, an even count, so ties keep their parity) moves min_i to -4 only
+    s16b, m16b, c16b, s8b, m8b = O.quant((x.astype(np.float32) - 2.0).astype(np.float16), O.MASK_K_BLOCK, 0.1)
+    assert int(m8b.ravel()[0]) == -4 and np.array_equal(s8b, s8)
     # dequant closed form
     d = O.dequant(s8b, m8b, c16b, O.MASK_K_BLOCK)
-    assert np.array_equal(d.reshape(-1)[:xs.size].astype(np.float32), (np.array([0, 0, 1, 2, 2, 2, 5, 9, 10]) - 3) * 0.5)
+    assert np.array_equal(d.reshape(-1)[:xs.size].astype(np.float32), (np.array([0, 0, 1, 2, 2, 2, 5, 9, 10]) - 4) * 0.5)
 
 
 def test_dequant_brute_force_against_torch():
