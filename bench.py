@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path: decode attention over a Huffman-compressed KV cache on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5] [--no-cpu-baseline]
+
+A step is one decode-attention pass of one layer over the whole compressed cache, already resident in HBM:
+fused decompress -> q.K^T, 1/sqrt(d) + softmax, fused decompress -> p.V, partial-sum reduce.  The printed value
+is compressed-cache bytes (payload + block_infos + thread_infos + min + 2*scale, i.e. the denominator of the
+reference's get_cr(), models/cache/kvcomp_encode.py:317-326, for K and V together) consumed per second.
+
+One JSON line goes to stdout; progress goes to stderr.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+
+# name -> shape and error bounds of the synthetic configurations
+WORKLOADS = {
+    # batch 1 Llama-2-7B layer, 4096 cached tokens
+    "cfg2": dict(B=1, H=32, Hq=32, D=128, T=4096, eb_k=0.1, eb_v=0.2, dist="gauss",
+                 desc="fused decode attention, Llama-2-7B layer: batch 1, 32 heads x 128, 4096 cached tokens, eb K 0.1 / V 0.2"),
+    # batched GQA, Mistral-7B-shaped
+    "cfg3": dict(B=16, H=8, Hq=32, D=128, T=8192, eb_k=0.1, eb_v=0.2, dist="gauss",
+                 desc="batched GQA decode attention, Mistral-7B layer: batch 16, 32 q / 8 kv heads x 128, 8192 cached tokens, eb K 0.1 / V 0.2"),
+    # long context, Phi-3-mini-shaped, heavy-tailed
+    "cfg5": dict(B=4, H=32, Hq=32, D=96, T=32768, eb_k=0.1, eb_v=0.3, dist="laplace",
+                 desc="long-context decode attention, Phi-3-mini layer: batch 4, 32 heads x 96, 32768 cached tokens, Laplace + 2% x50 outliers, eb K 0.1 / V 0.3"),
+}
+DEFAULT_WORKLOAD = "cfg3"
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def make_kv(cfg, device):
+    """Synthetic K/V [T, B, H, D] fp16 generated on the device (seeded)."""
+    import torch
+    T, B, H, D = cfg["T"], cfg["B"], cfg["H"], cfg["D"]
+    g = torch.Generator(device=device)
+    if cfg["dist"] == "gauss":
+        g.manual_seed(1234)
+        k = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32)
+        c = torch.exp(0.5 * torch.randn(H, D, generator=g, device=device, dtype=torch.float32))
+        g.manual_seed(1237)
+        for h in range(H):
+            c[h, torch.randperm(D, generator=g, device=device)[:4]] *= 20.0
+        k = (k * c).to(torch.float16)
+        g.manual_seed(1235)
+        v = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32).to(torch.float16)
+    else:
+        out = []
+        for seed in (1234, 1235):
+            g.manual_seed(seed)
+            u = torch.rand(T, B, H, D, generator=g, device=device, dtype=torch.float32) - 0.5
+            x = -torch.sign(u) * torch.log1p(-2.0 * u.abs().clamp(max=0.4999999))
+            m = torch.rand(T, B, H, D, generator=g, device=device) < 0.02
+            out.append(torch.where(m, x * 50.0, x).to(torch.float16))
+        k, v = out
+    return k, v
+
+
+def cpu_baseline(kctx, q, cfg, budget_s=12.0):
+    """The reference's fused K algorithm (bit-serial tree walk, fp16 dequantize, dot) restated in C
+    (oracle/kvc_oracle.c: kvo_fused_k_from_stream), timed on this host's cores over a bounded sample of
+    the same K stream."""
+    import numpy as np
+    from oracle import oracle as O
+    from kvcomp_amd.compute import dims_to_mask
+    B, H, D, T = cfg["B"], cfg["H"], cfg["D"], cfg["T"]
+    enc = kctx.encoded_data.cpu().numpy()
+    bi = kctx.block_infos.cpu().numpy()
+    ti = kctx.thread_infos.cpu().numpy()
+    tree = kctx.decode_codebook.cpu().numpy()
+    mn = kctx.quant_min_ints.cpu().numpy()
+    sc = kctx.quant_scales.cpu().numpy()
+    qh = q[:, ::cfg["Hq"] // H].contiguous().cpu().numpy()           # one query head per kv head
+    mask = dims_to_mask(kctx.quant_dims)
+    stride, rows, cols = B * H * D, T // 64, B * H
+    cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+    O.lib().kvo_set_threads(cores)
+
+    def run(nrows):
+        t0 = time.perf_counter()
+        O.fused_k_from_stream(enc, bi, ti, tree, mn, sc, qh, nrows * 64, stride, vec_len=D, mask=mask)
+        return time.perf_counter() - t0
+
+    def sample_bytes(nrows):
+        tiles = nrows * cols
+        payload = int(bi.view(np.uint32)[1::2][:tiles].astype(np.int64).sum())
+        per_group = D if mask == 0x1 else 1
+        groups = tiles * per_group if mask == 0x1 else nrows
+        return payload + tiles * 8 + tiles * 64 * 2 + groups * 3
+
+    probe = max(1, min(rows, 4))
+    dt = run(probe)
+    nrows = int(max(probe, min(rows, probe * budget_s / max(dt, 1e-6))))
+    dt = run(nrows)
+    return {"value": round(sample_bytes(nrows) / dt / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+            "sample": "fused K (tree-walk decode + fp16 dequant + dot) over the first %d of %d tokens of the same "
+                      "compressed K stream, %.1f s" % (nrows * 64, T, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py measures one GPU: this path shards by KV head or batch with no exchange, and no run here "
+            "uses a second GPU (--gpus %d refused)" % args.gpus)
+        sys.exit(2)
+
+    import torch
+    from kvcomp_amd.ctx import KVCompCtx, KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
+    from kvcomp_amd import attention as A
+
+    cfg = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, H, Hq, D, T = cfg["B"], cfg["H"], cfg["Hq"], cfg["D"], cfg["T"]
+    KVCompCacheConfigStatic.config = KVCompCacheConfig(args.workload, QuantMode.ChannelQuant, QuantMode.TokenQuant,
+                                                       64, 128, 64, 128, cfg["eb_k"], cfg["eb_v"])
+    log("[bench] %s" % cfg["desc"])
+    k, v = make_kv(cfg, dev)
+    kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    kctx.store(k)
+    vctx.store(v)
+    torch.cuda.synchronize()
+    t_store = time.perf_counter() - t0
+    del k, v
+    assert kctx.compressed_ctx_len == T and vctx.compressed_ctx_len == T
+    kb, vb = kctx.compressed_bytes(), vctx.compressed_bytes()
+    numel = T * B * H * D
+    log("[bench] compressed: K %.1f MB (CR %.2f, %.2f bits/sym)  V %.1f MB (CR %.2f, %.2f bits/sym); first store "
+        "(incl. codebook) %.1f ms" % (kb / 1e6, kctx.get_cr(), 8 * kctx.encoded_data.numel() / numel, vb / 1e6,
+                                      vctx.get_cr(), 8 * vctx.encoded_data.numel() / numel, t_store * 1e3))
+
+    g = torch.Generator(device=dev).manual_seed(1236)
+    q = torch.randn(B, Hq, D, generator=g, device=dev, dtype=torch.float32).to(torch.float16)
+    attn = A.CompressedAttention(kctx, vctx)
+
+    for _ in range(args.warmup):
+        attn.attend(q)
+    torch.cuda.synchronize()
+    prof = {"k": [], "v": []}
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        out = attn.attend(q, prof=prof)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    k_ms = sum(a.elapsed_time(b) for a, b in prof["k"]) / len(prof["k"])
+    v_ms = sum(a.elapsed_time(b) for a, b in prof["v"]) / len(prof["v"])
+    log("[bench] step %.3f ms; fused K kernel %.3f ms (%.1f GB/s compressed), fused V kernel %.3f ms (%.1f GB/s compressed)"
+        % (ms_per_step, k_ms, kb / k_ms / 1e6, v_ms, vb / v_ms / 1e6))
+    assert torch.isfinite(out).all()
+
+    dom, dom_ms, dom_bytes = ("kvc_fused_k_kernel", k_ms, kb) if k_ms >= v_ms else ("kvc_fused_v_kernel", v_ms, vb)
+    achieved = dom_bytes / dom_ms / 1e6
+    value = (kb + vb) / (ms_per_step * 1e-3) / 1e9
+    result = {
+        "metric": "fused decompress-matvec GB/s (% HBM peak); Huffman enc/dec GB/s; comp ratio",
+        "value": round(value, 3), "unit": "GB/s (compressed-cache bytes consumed per second by one decode-attention pass)",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 symbols, fp32 accumulate",
+        "data": "synthetic", "config": {"workload": "%s: %s" % (args.workload, cfg["desc"]),
+                                        "k_quant": "per-channel, 64-token blocks", "v_quant": "per-token",
+                                        "compressed_bytes": {"k": kb, "v": vb}, "fp16_bytes_per_tensor": 2 * numel,
+                                        "compression_ratio": {"k": round(kctx.get_cr(), 3), "v": round(vctx.get_cr(), 3)},
+                                        "fp16_equivalent_GBs": round(4 * numel / (ms_per_step * 1e-3) / 1e9, 1),
+                                        "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+                                        "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)}},
+        "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        log("[bench] timing the CPU restatement of the reference's fused K path ...")
+        result["cpu_baseline"] = cpu_baseline(kctx, q, cfg)
+    else:
+        result["cpu_baseline"] = None
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -88,10 +88,25 @@ class CompressedAttention:
             self._v_lut, self._v_lut_src = build_lut(self.v.decode_codebook), self.v.decode_codebook
         return self._k_lut, self._v_lut
 
-    def attend(self, q: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
+    @staticmethod
+    def _bracket(prof, key):
+        if prof is None:
+            return None
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        prof[key].append((a, b))
+        a.record()
+        return b
+
+    @staticmethod
+    def _bracket_end(ev):
+        if ev is not None:
+            ev.record()
+
+    def attend(self, q: torch.Tensor, scale: Optional[float] = None, prof: Optional[dict] = None) -> torch.Tensor:
         """q fp16 [B, Hq, D] -> fp32 [B, Hq, D].  Covers every stored token: the compressed part through the
         fused kernels, the fp16 tails (K and V compress on different block sizes, so their tails differ)
-        through dense matvecs."""
+        through dense matvecs.  `prof`, if given, collects (start, end) event pairs recorded on the launch
+        stream around the two fused kernels under the keys "k" and "v"."""
         B, Hq, D = q.shape
         rep = Hq // self.k.head_num
         scale = scale if scale is not None else 1.0 / math.sqrt(D)
@@ -101,7 +116,9 @@ class CompressedAttention:
         kc, vc = self.k.compressed_ctx_len, self.v.compressed_ctx_len
         parts = []
         if kc:
+            ev = self._bracket(prof, "k")
             parts.append(k_scores(self.k, k_lut, q)[0])
+            self._bracket_end(ev)
         if kc != T:
             tail = self.k.buffer.float().repeat_interleave(rep, dim=2)                  # [t, B, Hq, D]
             parts.append(torch.einsum("tbhd,bhd->bht", tail, q.float()))
@@ -109,7 +126,10 @@ class CompressedAttention:
         p = torch.softmax(scores * scale, dim=-1)
         out = torch.zeros(B, Hq, D, dtype=torch.float32, device=q.device)
         if vc:
-            part, _ = v_partials(self.v, v_lut, p[:, :, :vc].to(torch.float16).contiguous())
+            p16 = p[:, :, :vc].to(torch.float16).contiguous()
+            ev = self._bracket(prof, "v")
+            part, _ = v_partials(self.v, v_lut, p16)
+            self._bracket_end(ev)
             out += part.sum(dim=0)
         if vc != T:
             tail = self.v.buffer.float().repeat_interleave(rep, dim=2)

@@ -32,6 +32,10 @@
 #include <string.h>
 #include <math.h>
 
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
 #define KVO_VEC_PER_TILE 64   /* include/kernels.h:13,18  K_VEC_PER_BLK = V_VEC_PER_BLK = 64 */
 
 /* ------------------------------------------------------------------------------------------ */
@@ -572,13 +576,13 @@ void kvo_fused_v(const uint8_t *sym, const int8_t *min_i8, const uint16_t *scale
 /* ------------------------------------------------------------------------------------------ */
 /* CPU baseline leg: the reference's fused K path end to end on the host, as its kernel does    */
 /* it per lane -- bit-serial tree walk straight out of the payload, fp16 dequantize, dot with   */
-/* q -- (src/kernels.cu:293-348,721-776), with an fp32 accumulator.  One (min, scale) per       */
-/* 64-token block (kernels.cu:771-772).  score fp32 [B*H, T].  Returns 0 or a negative vector   */
-/* index on a malformed stream.                                                                */
+/* q -- (src/kernels.cu:293-348,721-776), with an fp32 accumulator.  mask 0xF: one (min, scale)  */
+/* per 64-token block (kernels.cu:771-772); mask 0x1: one per (block, b, h, channel).           */
+/* score fp32 [B*H, T].  Returns 0 or a negative vector index on a malformed stream.            */
 /* ------------------------------------------------------------------------------------------ */
 int64_t kvo_fused_k_from_stream(const uint8_t *encoded, const uint8_t *block_infos, const uint8_t *thread_infos,
                                 const uint8_t *tree, int64_t tree_bytes,
-                                const int8_t *min_i8, const uint16_t *scale_f16,
+                                const int8_t *min_i8, const uint16_t *scale_f16, int mask,
                                 const uint16_t *q, int64_t tokens, int64_t stride, int vec_len, float *score)
 {
     int64_t cols = stride / vec_len, rows = tokens / KVO_VEC_PER_TILE, tiles = rows * cols;
@@ -589,8 +593,9 @@ int64_t kvo_fused_k_from_stream(const uint8_t *encoded, const uint8_t *block_inf
     for (int64_t tau = 0; tau < tiles; tau++) {
         int64_t row = tau / cols, col = tau % cols;
         uint32_t off = kvo_rd32(block_infos + 8 * (size_t)tau);
-        int mn = min_i8[row];
-        float sc = kvo_h2f(scale_f16[row]);
+        const int per_channel = (mask == 0x1);
+        const int8_t *mnp = per_channel ? min_i8 + tau * vec_len : min_i8 + row;
+        const uint16_t *scp = per_channel ? scale_f16 + tau * vec_len : scale_f16 + row;
         for (int t = 0; t < KVO_VEC_PER_TILE; t++) {
             size_t v = (size_t)(tau * KVO_VEC_PER_TILE + t);
             uint16_t ti = (uint16_t)(thread_infos[2 * v] | (thread_infos[2 * v + 1] << 8));
@@ -606,6 +611,8 @@ int64_t kvo_fused_k_from_stream(const uint8_t *encoded, const uint8_t *block_inf
                 if (idx < 0 || idx >= tree_nodes) { rc = -(1 + (int64_t)v); break; }
                 if (tree[3 * idx]) {
                     if (n < vec_len) {
+                        int mn = per_channel ? mnp[n] : mnp[0];
+                        float sc = kvo_h2f(per_channel ? scp[n] : scp[0]);
                         float kv = kvo_h2f(kvo_f2h((float)((int)tree[3 * idx + 1] + mn) * sc));
                         acc += kv * kvo_h2f(q[col * vec_len + n]);
                     }
@@ -617,4 +624,16 @@ int64_t kvo_fused_k_from_stream(const uint8_t *encoded, const uint8_t *block_inf
         }
     }
     return rc;
+}
+
+/* Thread count of the CPU baseline leg (OpenMP over tiles); returns the count in effect. */
+int kvo_set_threads(int n)
+{
+#ifdef _OPENMP
+    if (n > 0) omp_set_num_threads(n);
+    return omp_get_max_threads();
+#else
+    (void)n;
+    return 1;
+#endif
 }

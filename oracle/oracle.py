@@ -239,7 +239,8 @@ def fused_v(sym_tbhd, min_i8, scale_f16, mask, block_size, p):
     return out
 
 
-def fused_k_from_stream(encoded, block_infos, thread_infos, tree, min_i8, scale_f16, q, tokens, stride, vec_len=128):
+def fused_k_from_stream(encoded, block_infos, thread_infos, tree, min_i8, scale_f16, q, tokens, stride, vec_len=128,
+                        mask=MASK_K_BLOCK, threads=None):
     """CPU baseline: the reference's fused K kernel per lane on the host (bit-serial walk, fp16 dequant, dot).
     Returns float32 [stride/vec_len, tokens]."""
     enc = np.ascontiguousarray(encoded, dtype=np.uint8)
@@ -248,9 +249,11 @@ def fused_k_from_stream(encoded, block_infos, thread_infos, tree, min_i8, scale_
     mn = np.ascontiguousarray(min_i8, dtype=np.int8).ravel()
     sc = np.ascontiguousarray(scale_f16, dtype=np.float16).ravel()
     out = np.zeros((stride // vec_len, tokens), np.float32)
+    if threads:
+        lib().kvo_set_threads(C.c_int(int(threads)))
     rc = lib().kvo_fused_k_from_stream(_p(enc), _p(np.ascontiguousarray(block_infos)),
                                        _p(np.ascontiguousarray(thread_infos)), _p(tree), _i64(tree.shape[0]),
-                                       _p(mn), _p(sc.view(np.uint16)), _p(q.view(np.uint16)), _i64(tokens),
+                                       _p(mn), _p(sc.view(np.uint16)), C.c_int(mask), _p(q.view(np.uint16)), _i64(tokens),
                                        _i64(stride), C.c_int(vec_len), _p(out))
     if rc != 0:
         raise ValueError("malformed stream at vector %d" % (-rc - 1))
