@@ -28,6 +28,10 @@ constexpr int KVC_STAGE_WORDS = KVC_STAGE_BYTES / 4;
 //   long[ ]  codes longer than lbits: {code left-aligned in 32 bits, len | sym << 8}
 //   entry[ ] 1 << lbits words indexed by the next lbits stream bits: len | sym << 8, or 0 when the
 //            code is longer than lbits (search long[]) or the bits match no code.
+//   fentry[] same index, for the fused kernels: the symbol as an fp32 bit pattern with (32 - len) & 31 in
+//            its five lowest mantissa bits (zero for any integer <= 255, so the value read as a float is
+//            the symbol to within 4e-6 relative, and read as a shift count it is a rotate-left by len).
+//            Indices whose code is longer than lbits or that match no code hold "symbol 0, length 1".
 //   group    how many symbols may be decoded from one 32-bit window: floor(32 / lmax), one of 8,4,2,1.
 // ---------------------------------------------------------------------------------------------------
 constexpr int KVC_LUT_MAX_BITS = 10;
@@ -35,8 +39,9 @@ constexpr int KVC_LUT_MAX_LONG = 256;
 constexpr int KVC_LUT_HEADER_WORDS = 4;
 constexpr int KVC_LUT_LONG_WORDS = 2 * KVC_LUT_MAX_LONG;
 constexpr int KVC_LUT_ENTRY_WORDS = 1 << KVC_LUT_MAX_BITS;
-constexpr int KVC_LUT_WORDS = KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS + KVC_LUT_ENTRY_WORDS;
-constexpr int KVC_LUT_BYTES = KVC_LUT_WORDS * 4;          // 6160
+constexpr int KVC_LUT_FENTRY_OFFSET = KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS + KVC_LUT_ENTRY_WORDS;
+constexpr int KVC_LUT_WORDS = KVC_LUT_FENTRY_OFFSET + KVC_LUT_ENTRY_WORDS;
+constexpr int KVC_LUT_BYTES = KVC_LUT_WORDS * 4;          // 10256
 constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2, rounded up
 
 // ---------------------------------------------------------------------------------------------------

@@ -107,12 +107,13 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
             cur = s_child[(idx >> (lbits - 1 - depth)) & 1u][cur];
         }
         entries[idx] = e;
+        const uint32_t len = e & 0xffu, sym = e >> 8;
+        lut[KVC_LUT_FENTRY_OFFSET + idx] = len ? (__float_as_uint((float)sym) | ((32u - len) & 31u)) : 31u;
     }
     __syncthreads();
     if (tid == 0) {
         uint32_t nlong = s_nlong < (uint32_t)KVC_LUT_MAX_LONG ? s_nlong : (uint32_t)KVC_LUT_MAX_LONG;
         uint32_t group = lmax <= 4 ? 8u : lmax <= 8 ? 4u : lmax <= 16 ? 2u : 1u;
-        if (nlong > 0 && lmax > 16) group = 1u;
         lut[0] = lbits;
         lut[1] = lmax;
         lut[2] = nlong;

@@ -10,6 +10,8 @@
 #pragma once
 #include "kvc_common.h"
 
+#include <cstdlib>
+
 struct KvcStreamArgs {
     const uint8_t *enc;            // concatenated tile payloads
     int64_t enc_bytes;
@@ -124,3 +126,63 @@ __device__ __forceinline__ void kvc_dispatch_group(const uint32_t *s_lut, Body &
         else body.template operator()<1, true>();
     }
 }
+
+// ---------------------------------------------------------------------------------------------------
+// host side: geometry checks and launch shape shared by the decoders
+// ---------------------------------------------------------------------------------------------------
+static inline int kvc_tiles_per_wave(int64_t tiles)
+{
+    static int forced = -1;
+    if (forced < 0) {
+        const char *e = std::getenv("KVC_TILES_PER_WAVE");
+        forced = e ? std::atoi(e) : 0;
+    }
+    if (forced > 0) return forced;
+    return tiles >= 32768 ? 2 : 1;
+}
+
+static inline int kvc_fill_stream_args(KvcStreamArgs &s, const uint8_t *d_encoded, int64_t encoded_bytes,
+                                const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                                const uint8_t *d_thread_infos, int64_t thread_infos_bytes, const uint32_t *d_luts,
+                                int is_k, int64_t tokens, int64_t stride, int64_t head_dim, int64_t *rows_out)
+{
+    KVC_REQUIRE(head_dim > 0 && head_dim <= KVC_K_VEC_LEN && head_dim % 8 == 0, "head_dim must be a multiple of 8, <= 128");
+    KVC_REQUIRE(stride > 0 && stride % 4 == 0, "stride must be a positive multiple of 4");
+    int64_t rows, cols;
+    if (is_k) {
+        KVC_REQUIRE(tokens % KVC_K_VEC_PER_BLK == 0, "K: token count must be a multiple of 64");
+        KVC_REQUIRE(stride % head_dim == 0, "K: stride must be a multiple of head_dim");
+        rows = tokens / KVC_K_VEC_PER_BLK;
+        cols = stride / head_dim;
+    } else {
+        KVC_REQUIRE(tokens % KVC_V_VEC_LEN == 0, "V: token count must be a multiple of 128");
+        KVC_REQUIRE(stride % KVC_V_VEC_PER_BLK == 0, "V: stride must be a multiple of 64");
+        rows = tokens / KVC_V_VEC_LEN;
+        cols = stride / KVC_V_VEC_PER_BLK;
+    }
+    KVC_REQUIRE(rows <= 65535, "too many tile rows (%lld) for one launch", (long long)rows);
+    KVC_REQUIRE(block_infos_bytes == rows * cols * 8, "block_infos holds %lld bytes, geometry needs %lld",
+                (long long)block_infos_bytes, (long long)(rows * cols * 8));
+    KVC_REQUIRE(thread_infos_bytes == rows * cols * KVC_WAVE * 2, "thread_infos holds %lld bytes, geometry needs %lld",
+                (long long)thread_infos_bytes, (long long)(rows * cols * KVC_WAVE * 2));
+    KVC_REQUIRE(((uintptr_t)d_block_infos & 3) == 0 && ((uintptr_t)d_thread_infos & 1) == 0, "metadata pointers misaligned");
+    s.enc = d_encoded;
+    s.enc_bytes = encoded_bytes;
+    s.block_infos = d_block_infos;
+    s.thread_infos = reinterpret_cast<const uint16_t *>(d_thread_infos);
+    s.luts = d_luts;
+    s.rows_per_codebook = 0;
+    s.cols = (int)cols;
+    s.tiles_per_wave = kvc_tiles_per_wave(rows * cols);
+    s.vec_len = is_k ? (int)head_dim : KVC_V_TOKENS;
+    s.stride = stride;
+    *rows_out = rows;
+    return 0;
+}
+
+static inline dim3 kvc_grid(const KvcStreamArgs &s, int64_t rows)
+{
+    const int per_wg = KVC_WAVES_PER_WG * s.tiles_per_wave;
+    return dim3((unsigned)((s.cols + per_wg - 1) / per_wg), (unsigned)rows);
+}
+

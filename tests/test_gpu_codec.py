@@ -41,7 +41,7 @@ def _make_stream(x_tbhd, is_k, eb, mask, block_size, tree_format=3):
                 code=code, length=length, counts=counts)
 
 
-SHAPES = [(256, 1, 4, 128), (128, 2, 2, 128), (256, 1, 3, 64)]
+SHAPES = [(256, 1, 4, 128), (128, 2, 2, 128), (256, 1, 3, 64), (256, 2, 2, 96)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -89,7 +89,8 @@ def test_entropy_encode_matches_oracle(shape, is_k):
     assert idx[0] == ref_bi.size // 8 and idx[1] == ref_payload.size
 
 
-@pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((128, 2, 2, 128), 1), ((128, 2, 2, 128), 4), ((256, 1, 3, 64), 2)])
+@pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((128, 2, 2, 128), 1), ((128, 2, 2, 128), 4), ((256, 1, 3, 64), 2),
+                                       ((256, 2, 2, 96), 1), ((128, 1, 2, 96), 8)])
 @pytest.mark.parametrize("mask", [O.MASK_K_BLOCK, O.MASK_CHANNEL])
 def test_fused_k_matches_oracle(shape, rep, mask):
     T, B, H, D = shape
@@ -111,7 +112,8 @@ def test_fused_k_matches_oracle(shape, rep, mask):
     assert np.abs(got - ref32).max() <= 1e-3 * np.abs(ref32).max()
 
 
-@pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((256, 2, 2, 128), 1), ((256, 2, 2, 128), 4), ((128, 1, 3, 64), 2)])
+@pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((256, 2, 2, 128), 1), ((256, 2, 2, 128), 4), ((128, 1, 3, 64), 2),
+                                       ((256, 2, 2, 96), 1), ((128, 2, 4, 96), 2), ((128, 1, 2, 96), 8)])
 @pytest.mark.parametrize("mask", [O.MASK_V_TOKEN, O.MASK_SIM_TOKEN, O.MASK_VECTOR])
 def test_fused_v_matches_oracle(shape, rep, mask):
     T, B, H, D = shape
@@ -135,6 +137,35 @@ def test_fused_v_matches_oracle(shape, rep, mask):
 @pytest.mark.parametrize("mask", [O.MASK_K_BLOCK, O.MASK_V_TOKEN, O.MASK_CHANNEL, O.MASK_SIM_TOKEN, O.MASK_VECTOR, O.MASK_SIM_BLOCK])
 @pytest.mark.parametrize("eb", [0.03, 0.1, 0.13, 0.2])
 def test_quant_dequant_bit_exact(mask, eb):
+    _quant_dequant_case(mask, eb)
+
+
+@pytest.mark.parametrize("eb_k,eb_v", [(0.3, 0.45), (0.03, 0.05)])
+def test_fused_across_code_length_regimes(eb_k, eb_v):
+    """Short codes (8 symbols per window), and long codes (4 per window with the overflow check)."""
+    m = kc()
+    T, B, H, D = 256, 1, 4, 128
+    s = _make_stream(S.synth_k(T, B, H, D), True, eb_k, O.MASK_CHANNEL, 64)
+    q = S.synth_q(B, H, D)
+    ref = O.fused_k(s["sym"].reshape(T, B, H, D), s["mn"], s["scale"], O.MASK_CHANNEL, 64, S.np16(q))
+    out = torch.zeros(B, H, T, dtype=torch.float16, device=DEV)
+    m.k_decode_and_mat_vec_mul_cuda_export(_dev(s["dec"]), _dev(s["bi"]), _dev(s["ti"]), _dev(s["payload"]),
+                                           _dev(s["mn"].ravel()), _dev(s["scale"].ravel().view(np.uint16), torch.float16),
+                                           q.to(DEV), out, H, D)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= 1e-3 * np.abs(ref).max()
+    print("K lmax", int(s["length"].max()))
+    s = _make_stream(S.synth_v(T, B, H, D), False, eb_v, O.MASK_V_TOKEN, 128)
+    p = S.synth_p(B, H, T)
+    ref = O.fused_v(s["sym"].reshape(T, B, H, D), s["mn"], s["scale"], O.MASK_V_TOKEN, 128, S.np16(p))
+    part = torch.zeros(T // 128, B, H, D, dtype=torch.float16, device=DEV)
+    m.v_decode_and_mat_vec_mul_cuda_export(_dev(s["dec"]), _dev(s["bi"]), _dev(s["ti"]), _dev(s["payload"]),
+                                           _dev(s["mn"].ravel()), _dev(s["scale"].ravel().view(np.uint16), torch.float16),
+                                           p.to(DEV), part, H, D)
+    assert np.abs(part.float().sum(0).cpu().numpy() - ref).max() <= 1e-3 * np.abs(ref).max()
+    print("V lmax", int(s["length"].max()))
+
+
+def _quant_dequant_case(mask, eb):
     from kvcomp_amd import compute as cp
     T, B, H, D = 256, 2, 4, 128
     x = S.synth_k(T, B, H, D)
@@ -262,3 +293,37 @@ def test_errors_raise_instead_of_aborting():
         m.calculate_buffer_size(sym, True, 1, 128)
     with pytest.raises(RuntimeError):
         m.build_codebook([torch.zeros(100, dtype=torch.uint8, device=DEV)])   # a lone symbol has no usable code
+
+
+@pytest.mark.parametrize("is_k", [True, False])
+@pytest.mark.parametrize("nsym", [14, 22])
+def test_fused_with_long_codes_uses_slow_path(is_k, nsym):
+    """Codebooks whose codes exceed the table index: the fused kernels must fall back and still be right."""
+    rng = np.random.default_rng(8)
+    T, B, H, D = 256, 1, 2, 128
+    bs = 64 if is_k else 128
+    sym = _skewed_symbols((T // bs, bs, B, H, D), nsym, rng)
+    counts = np.bincount(sym.ravel(), minlength=256).astype(np.int64)
+    code, length = O.huffman_build(counts)
+    _, enc = O.encode_table(code, length, counts)
+    st, dec = O.decode_tree(code, length, counts)
+    payload, bi, ti = O.encode_tiles(sym, is_k, enc, 0)
+    mask = O.MASK_K_BLOCK if is_k else O.MASK_V_TOKEN
+    gs = O.group_shape(sym.shape, mask)
+    mn = rng.integers(-20, 5, size=gs).astype(np.int8)
+    scale = rng.uniform(0.05, 0.5, size=gs).astype(np.float16)
+    m = kc()
+    args = (_dev(dec), _dev(bi), _dev(ti), _dev(payload), _dev(mn.ravel()), _dev(scale.ravel().view(np.uint16), torch.float16))
+    if is_k:
+        q = S.synth_q(B, H, D)
+        ref = O.fused_k(sym.reshape(T, B, H, D), mn, scale, mask, bs, S.np16(q))
+        out = torch.zeros(B, H, T, dtype=torch.float16, device=DEV)
+        m.k_decode_and_mat_vec_mul_cuda_export(*args, q.to(DEV), out, H, D)
+        got = out.float().cpu().numpy()
+    else:
+        p = S.synth_p(B, H, T)
+        ref = O.fused_v(sym.reshape(T, B, H, D), mn, scale, mask, bs, S.np16(p))
+        part = torch.zeros(T // 128, B, H, D, dtype=torch.float16, device=DEV)
+        m.v_decode_and_mat_vec_mul_cuda_export(*args, p.to(DEV), part, H, D)
+        got = part.float().sum(0).cpu().numpy()
+    assert np.abs(got - ref).max() <= 1e-3 * np.abs(ref).max()
