@@ -31,7 +31,7 @@ struct KvcEncodeArgs {
     uint8_t *encoded;
     int64_t encoded_cap;
     uint32_t base_global_offset;
-    uint32_t *status;          // [0] total payload bytes, [1] error bits
+    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload
     uint32_t *idx_offset;      // {tiles, bytes}  (include/kernels.h:34-42)
 };
 
@@ -109,14 +109,16 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs 
 __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
 {
     __shared__ uint32_t s_wave[16];
-    __shared__ uint32_t s_carry;
+    __shared__ uint32_t s_carry, s_max;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) s_carry = 0;
+    if (tid == 0) { s_carry = 0; s_max = 0; }
+    uint32_t my_max = 0;
     __syncthreads();
     for (int64_t base = 0; base < a.tiles; base += 1024) {
         const int64_t tile = base + tid;
         uint32_t bn = 0;
         if (tile < a.tiles) bn = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile)[1] & 0xffffu;
+        my_max = bn > my_max ? bn : my_max;
         const uint32_t incl = kvc_wave_inclusive_scan(bn, lane);
         if (lane == KVC_WAVE - 1) s_wave[wave] = incl;
         __syncthreads();
@@ -127,9 +129,12 @@ __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
         if (tid == 1023) s_carry = before + incl;
         __syncthreads();
     }
+    atomicMax(&s_max, my_max);
+    __syncthreads();
     if (tid == 0) {
         const uint32_t total = s_carry;
         a.status[0] = total;
+        a.status[2] = s_max;
         if ((int64_t)total > a.encoded_cap) atomicOr(&a.status[1], KVC_ENC_ERR_CAPACITY);
         a.idx_offset[0] = (uint32_t)a.tiles;
         a.idx_offset[1] = total;
@@ -207,7 +212,8 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a
 static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, int64_t stride,
                               const uint8_t *d_encode_table, int64_t encode_table_bytes, uint8_t *d_block_infos,
                               uint8_t *d_thread_infos, uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
-                              uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes, void *stream_)
+                              uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes,
+                              int64_t *h_max_tile_bytes, void *stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     int64_t sizes[4];
@@ -245,8 +251,8 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     hipLaunchKernelGGL(kvc_encode_scan_kernel, dim3(1), dim3(1024), 0, stream, a);
     hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     KVC_HIP(hipGetLastError());
-    uint32_t h_status[2] = {0, 0};
-    KVC_HIP(hipMemcpyAsync(h_status, slot, 8, hipMemcpyDeviceToHost, stream));
+    uint32_t h_status[3] = {0, 0, 0};
+    KVC_HIP(hipMemcpyAsync(h_status, slot, 12, hipMemcpyDeviceToHost, stream));
     KVC_HIP(hipStreamSynchronize(stream));   // the reference returns after cudaDeviceSynchronize (kernels.cu:957)
     if (h_status[1] & KVC_ENC_ERR_NO_CODE) return kvc_fail(-3, "a symbol has no code in the encode table");
     if (h_status[1] & KVC_ENC_ERR_TILE_TOO_BIG)
@@ -254,6 +260,7 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     if (h_status[1] & KVC_ENC_ERR_CAPACITY)
         return kvc_fail(-3, "payload (%u bytes) does not fit the encoded_data buffer (%lld bytes)", h_status[0], (long long)encoded_cap);
     *h_total_bytes = h_status[0];
+    if (h_max_tile_bytes) *h_max_tile_bytes = h_status[2];
     return 0;
 }
 
@@ -261,20 +268,22 @@ extern "C" int kvc_k_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_
                                     int64_t encode_table_bytes, uint8_t *d_block_infos, uint8_t *d_thread_infos,
                                     uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                                     uint32_t base_global_offset, int64_t head_num, int64_t head_dim,
-                                    int64_t *h_total_bytes, void *stream)
+                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, void *stream)
 {
     (void)head_num;
     return kvc_entropy_encode(1, d_sym, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
-                              d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes, stream);
+                              d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
+                              h_max_tile_bytes, stream);
 }
 
 extern "C" int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride, const uint8_t *d_encode_table,
                                     int64_t encode_table_bytes, uint8_t *d_block_infos, uint8_t *d_thread_infos,
                                     uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                                     uint32_t base_global_offset, int64_t head_num, int64_t head_dim,
-                                    int64_t *h_total_bytes, void *stream)
+                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, void *stream)
 {
     (void)head_num;
     return kvc_entropy_encode(0, d_sym, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
-                              d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes, stream);
+                              d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
+                              h_max_tile_bytes, stream);
 }

@@ -344,14 +344,17 @@ static void kvc_launch_fused(int is_k, const KvcFusedArgs &a, dim3 grid, size_t 
 
 // LDS words per wave for the staged payload: room for about twice the average tile (tiles that still do
 // not fit are decoded from global memory), between 1 KiB and the largest tile the format allows.
-static int kvc_pick_stage_words(int64_t encoded_bytes, int64_t tiles)
+static int kvc_pick_stage_words(int64_t encoded_bytes, int64_t tiles, int64_t max_tile_bytes)
 {
     static int forced = -1;
     if (forced < 0) {
         const char *e = std::getenv("KVC_STAGE_BYTES");
         forced = e ? std::atoi(e) : 0;
     }
-    int64_t bytes = forced > 0 ? forced : 2 * (encoded_bytes / (tiles > 0 ? tiles : 1)) + 64;
+    // payload + up to 15 bytes before it in its first chunk, rounded up to chunks, + lead and look-ahead words
+    int64_t bytes = max_tile_bytes > 0 ? ((max_tile_bytes + 15 + 15) / 16) * 16 + 4 * (KVC_STAGE_LEAD_WORDS + 2)
+                                       : 2 * (encoded_bytes / (tiles > 0 ? tiles : 1)) + 64;
+    if (forced > 0) bytes = forced;
     const int64_t max_bytes = ((KVC_MAX_TILE_BYTES + 15 + 15) / 16) * 16 + 16 * KVC_STAGE_LEAD_WORDS / 4 + 16;
     if (bytes < 1024) bytes = 1024;
     if (bytes > max_bytes) bytes = max_bytes;
@@ -365,7 +368,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                      const int8_t *d_min, const void *d_scale, int quant_mask, const void *d_x, void *d_out,
                      int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                      float *elapsed_ms, void *stream_, const uint32_t *d_luts = nullptr, int rows_per_codebook = 0,
-                     int out_f32 = 0)
+                     int out_f32 = 0, int64_t max_tile_bytes = 0)
 {
     hipStream_t stream = (hipStream_t)stream_;
     if (tokens == 0) {
@@ -405,7 +408,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     a.kv_heads = (int)kv_heads;
     a.q_heads = (int)q_heads;
     a.head_dim = (int)head_dim;
-    a.stage_words = kvc_pick_stage_words(encoded_bytes, rows * a.s.cols);
+    a.stage_words = kvc_pick_stage_words(encoded_bytes, rows * a.s.cols, max_tile_bytes);
     const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
     const size_t lds = (size_t)KVC_WAVES_PER_WG * (size_t)(slots * 128 * rep + a.stage_words) * 4;   // operand tables + staging
     KvcTimer timer(elapsed_ms, stream);
@@ -469,26 +472,26 @@ extern "C" int kvc_k_scores_lut(const void *d_luts, int64_t rows_per_codebook, c
                                 int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                                 const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                                 const void *d_quant_scales_f16, int quant_mask, const void *d_q_f16, void *d_scores,
-                                int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
-                                int64_t head_dim, float *elapsed_ms, void *stream)
+                                int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
+                                int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream)
 {
     KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
     return kvc_fused(1, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
                      d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_q_f16, d_scores, tokens,
                      batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
-                     (int)rows_per_codebook, out_f32);
+                     (int)rows_per_codebook, out_f32, max_tile_bytes);
 }
 
 extern "C" int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
                                   int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                                   const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                                   const void *d_quant_scales_f16, int quant_mask, const void *d_p_f16, void *d_partial,
-                                  int out_f32, int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads,
-                                  int64_t head_dim, float *elapsed_ms, void *stream)
+                                  int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
+                                  int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream)
 {
     KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
     return kvc_fused(0, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
                      d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_p_f16, d_partial, tokens,
                      batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
-                     (int)rows_per_codebook, out_f32);
+                     (int)rows_per_codebook, out_f32, max_tile_bytes);
 }

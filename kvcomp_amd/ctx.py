@@ -165,6 +165,7 @@ class KVCompCtx:
         self._min_ints = _Growable()
         self._scales = _Growable()
         self.buffer: Optional[torch.Tensor] = None
+        self.max_tile_bytes = 0          # largest tile payload seen so far (sizes the fused decoders' LDS staging)
         self.encode_codebook: Optional[torch.Tensor] = None
         self.decode_codebook: Optional[torch.Tensor] = None
 
@@ -214,6 +215,7 @@ class KVCompCtx:
         fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
         encoded_, block_infos_, vec_infos_ = fn(quant_ints, self.encode_codebook, bi_buf, ti_buf, idx_buf, payload_buf,
                                                 self._encoded.used, self.head_num, self.head_dim)
+        self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
         self._encoded.append(encoded_)
         self._block_infos.append(block_infos_)
         self._thread_infos.append(vec_infos_)
