@@ -193,6 +193,11 @@ int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const void *d_scal
                 int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
                 void *d_out_f16, void *stream);
 
+/* ---- measurement aid (no counterpart in the reference) ----------------------------------------------
+ * Plain device-to-device copy of `bytes` bytes (a multiple of 16) by a grid-stride kernel named
+ * kvc_calibration_copy_kernel: a dispatch of exactly known HBM traffic to scale profiler counters by. */
+int kvc_calibration_copy(void *d_dst, const void *d_src, int64_t bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -389,3 +389,24 @@ extern "C" int kvc_k_mat_vec_mul(const void *d_k_f16, const void *d_q_f16, void 
     KVC_HIP(hipGetLastError());
     return timer.finish();
 }
+
+// ---------------------------------------------------------------------------------------------------
+// plain device-to-device copy of a known size: the yardstick that the HBM traffic counters
+// (FETCH_SIZE / WRITE_SIZE) are scaled against when a profile of this library is read.
+// ---------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(KVC_WG) kvc_calibration_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n16)
+{
+    for (int64_t i = (int64_t)blockIdx.x * KVC_WG + threadIdx.x; i < n16; i += (int64_t)gridDim.x * KVC_WG) dst[i] = src[i];
+}
+
+extern "C" int kvc_calibration_copy(void *d_dst, const void *d_src, int64_t bytes, void *stream_)
+{
+    KVC_REQUIRE(bytes >= 0 && bytes % 16 == 0, "size must be a multiple of 16");
+    KVC_REQUIRE(((uintptr_t)d_dst & 15) == 0 && ((uintptr_t)d_src & 15) == 0, "pointers must be 16-byte aligned");
+    if (bytes == 0) return 0;
+    int64_t wgs = (bytes / 16 + KVC_WG - 1) / KVC_WG;
+    if (wgs > 8192) wgs = 8192;
+    hipLaunchKernelGGL(kvc_calibration_copy_kernel, dim3((unsigned)wgs), dim3(KVC_WG), 0, (hipStream_t)stream_,
+                       reinterpret_cast<const uint4 *>(d_src), reinterpret_cast<uint4 *>(d_dst), bytes / 16);
+    return kvc_check_hip(hipGetLastError(), "kvc_calibration_copy_kernel launch");
+}
