@@ -58,6 +58,12 @@ extern "C" {
 
 const char *kvc_last_error(void);
 int kvc_abi_version(void);
+/* Tuning knobs (no counterpart in the reference).  Each can also be preset through the environment
+ * variable KVCOMP_<NAME IN CAPITALS>, read once on first use.
+ *   "fused_rows":           -1 (default) the fused decoders decide per call whether to re-lay a tile's lane
+ *                           streams as LDS rows; 0 never; 1 whenever the rows fit.
+ *   "fused_tiles_per_wave":  0 (default) chosen per call; n > 0: consecutive tiles one wave works through. */
+int kvc_set_option(const char *name, int value);
 
 /* ---- sizes: calculate_buffer_size (kernels.cu:893-917) --------------------------------------------
  * out4 = {block_infos bytes, thread_infos bytes, idx_offset bytes (8), payload pre-allocation bytes}. */
@@ -82,20 +88,21 @@ int kvc_build_codebook_host(const int64_t *h_counts256, int tree_format, int *sh
  * returning, like the reference's cudaDeviceSynchronize.  d_idx_offset (8 B) receives
  * {u32 tiles, u32 bytes} as in include/kernels.h:34-42.  block_info.offset = base_global_offset +
  * offset inside this call's payload.  Fails if a tile payload exceeds 8191 B (thread_info is u16) or
- * the payload exceeds encoded_cap.  *h_max_tile_bytes (may be NULL) receives the largest tile payload
- * of this call, which the table-driven fused decoders accept as a sizing hint. */
+ * the payload exceeds encoded_cap.  *h_max_tile_bytes / *h_max_stream_bytes (each may be NULL) receive the
+ * largest tile payload and the longest single lane stream of this call, which the table-driven fused
+ * decoders accept as sizing hints. */
 int kvc_k_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride,
                          const uint8_t *d_encode_table, int64_t encode_table_bytes,
                          uint8_t *d_block_infos, uint8_t *d_thread_infos, uint8_t *d_idx_offset,
                          uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
-                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes, int64_t *h_max_tile_bytes,
-                         void *stream);
+                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes,
+                         int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream);
 int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride,
                          const uint8_t *d_encode_table, int64_t encode_table_bytes,
                          uint8_t *d_block_infos, uint8_t *d_thread_infos, uint8_t *d_idx_offset,
                          uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
-                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes, int64_t *h_max_tile_bytes,
-                         void *stream);
+                         int64_t head_num, int64_t head_dim, int64_t *h_total_bytes,
+                         int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream);
 
 /* ---- decode: k_/v_entropy_decode_cuda_export (kernels.cu:1013-1087) -------------------------------
  * d_out uint8 [tokens, stride].  If elapsed_ms != NULL the kernel is bracketed by events, the call
@@ -150,8 +157,13 @@ int kvc_v_decode_and_mat_vec_mul(const uint8_t *d_decode_tree, int64_t decode_tr
  *   kvc_k_scores_lut / kvc_v_partials_lut: as kvc_k_/v_decode_and_mat_vec_mul, plus
  *     rows_per_codebook: tile rows (64 tokens for K, 128 for V) that share one table; 0 = one table for all
  *     out_f32:           1 writes fp32 results instead of fp16
- *     max_tile_bytes:    largest tile payload in the stream (from the encoder), 0 = unknown.  It only sizes
- *                        the per-wave LDS staging area; tiles that do not fit are decoded from global memory. */
+ *     max_tile_bytes, max_stream_bytes:
+ *                        largest tile payload / longest lane stream in the payload (from the encoder),
+ *                        0 = unknown.  They only size the LDS staging; tiles that exceed them are decoded
+ *                        from global memory.
+ *     max_code_bits:     longest code of the codebook(s), 0 = unknown.  It only sizes the table kept in LDS
+ *                        (fewer bytes, more waves per CU); a codebook with longer codes than stated still
+ *                        decodes correctly, on the slow path. */
 int64_t kvc_lut_bytes(void);
 int kvc_build_lut(const uint8_t *d_decode_trees, int64_t tree_bytes, int tree_format, int64_t n_codebooks,
                   int64_t tree_stride_bytes, void *d_luts, void *stream);
@@ -159,14 +171,16 @@ int kvc_k_scores_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_
                      int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                      const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                      const void *d_quant_scales_f16, int quant_mask, const void *d_q_f16, void *d_scores,
-                     int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
-                     int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream);
+                     int out_f32, int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits,
+                     int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                     float *elapsed_ms, void *stream);
 int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
                        int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                        const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                        const void *d_quant_scales_f16, int quant_mask, const void *d_p_f16, void *d_partial,
-                       int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
-                       int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream);
+                       int out_f32, int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits,
+                       int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                       float *elapsed_ms, void *stream);
 
 /* ---- dense baseline: k_mat_vec_mul_cuda_export (kernels.cu:1182-1273) ------------------------------
  * d_k fp16 [tokens, batch, heads, head_dim], d_q fp16 [batch, heads, head_dim],

@@ -15,11 +15,12 @@ _i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
 # name -> argtypes (every function returns int unless listed in _RESTYPES)
 _SIGNATURES = {
     "kvc_abi_version": [],
+    "kvc_set_option": [C.c_char_p, _int],
     "kvc_calculate_buffer_size": [_i64, _i64, _int, _i64, _i64, _i64p],
     "kvc_histogram": [_vp, _i64, _vp, _vp],
     "kvc_build_codebook_host": [_i64p, _int, _intp, _vp, _i64, _i64p, _vp, _i64, _i64p],
-    "kvc_k_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _vp],
-    "kvc_v_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _vp],
+    "kvc_k_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
+    "kvc_v_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
     "kvc_k_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_k_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,
@@ -28,10 +29,10 @@ _SIGNATURES = {
                                      _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_lut_bytes": [],
     "kvc_build_lut": [_vp, _i64, _int, _i64, _i64, _vp, _vp],
-    "kvc_k_scores_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64,
-                         _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
-    "kvc_v_partials_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64,
-                           _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_k_scores_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64,
+                         _int, _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_v_partials_lut": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp, _int, _i64, _i64,
+                           _int, _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_k_mat_vec_mul": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_quant_groups": [_i64, _i64, _i64, _i64, _i64, _int],
     "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],

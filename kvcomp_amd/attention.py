@@ -51,6 +51,7 @@ def k_scores(ctx: KVCompCtx, lut: torch.Tensor, q: torch.Tensor, out: Optional[t
             _ptr(lut), 0, _ptr(ctx.block_infos), ctx.block_infos.numel(), _ptr(ctx.thread_infos), ctx.thread_infos.numel(),
             _ptr(ctx.encoded_data), ctx.encoded_data.numel(), _ptr(ctx.quant_min_ints), _ptr(ctx.quant_scales),
             dims_to_mask(ctx.quant_dims), _ptr(q), _ptr(out), 1 if out.dtype == torch.float32 else 0, ctx.max_tile_bytes,
+            ctx.max_stream_bytes, ctx.max_code_bits,
             ctx.compressed_ctx_len, B, ctx.head_num, Hq, D, C.byref(ms) if timed else None, _stream(q.device)))
     return out, float(ms.value)
 
@@ -67,6 +68,7 @@ def v_partials(ctx: KVCompCtx, lut: torch.Tensor, p: torch.Tensor, out: Optional
             _ptr(lut), 0, _ptr(ctx.block_infos), ctx.block_infos.numel(), _ptr(ctx.thread_infos), ctx.thread_infos.numel(),
             _ptr(ctx.encoded_data), ctx.encoded_data.numel(), _ptr(ctx.quant_min_ints), _ptr(ctx.quant_scales),
             dims_to_mask(ctx.quant_dims), _ptr(p), _ptr(out), 1 if out.dtype == torch.float32 else 0, ctx.max_tile_bytes,
+            ctx.max_stream_bytes, ctx.max_code_bits,
             T, B, ctx.head_num, Hq, ctx.head_dim, C.byref(ms) if timed else None, _stream(p.device)))
     return out, float(ms.value)
 

@@ -24,30 +24,39 @@ constexpr int KVC_STAGE_WORDS = KVC_STAGE_BYTES / 4;
 // ---------------------------------------------------------------------------------------------------
 // decode look-up table (built on the device from the decode tree, see kvc_lut.hip)
 //
-//   header   {lbits, lmax, n_long, group}
+//   header   {lbits, lmax, n_long, group, fused_group, fused_check, 0, 0}
 //   long[ ]  codes longer than lbits: {code left-aligned in 32 bits, len | sym << 8}
 //   entry[ ] 1 << lbits words indexed by the next lbits stream bits: len | sym << 8, or 0 when the
 //            code is longer than lbits (search long[]) or the bits match no code.
-//   fentry[] same index, for the fused kernels: the symbol as an fp32 bit pattern with (32 - len) & 31 in
-//            its five lowest mantissa bits (zero for any integer <= 255, so the value read as a float is
-//            the symbol to within 4e-6 relative, and read as a shift count it is a rotate-left by len).
-//            Indices whose code is longer than lbits or that match no code hold "symbol 0, length 1".
+//   fentry[] for the fused kernels, indexed by the next lbits stream bits taken least-significant-bit first
+//            (bit j of the index = j-th next stream bit): the symbol as an fp32 bit pattern with the code
+//            length in its lowest mantissa byte (zero for any integer <= 255, so read as a float the entry
+//            is the symbol to within 4e-6 relative, read as a shift count it is the length).  Indices
+//            whose code is longer than lbits or that match no code hold "symbol 0, length 1".
 //   group    how many symbols may be decoded from one 32-bit window: floor(32 / lmax), one of 8,4,2,1.
+//   fused_group / fused_check
+//            the same for the fused kernels, whose window has 30 usable bits: 8 if lmax <= 3, 4 if
+//            lmax <= 7 (both guaranteed to fit); for longer codes 4 with fused_check = 1 when four symbols
+//            are expected to stay well inside the window (mean code length, estimated from the code
+//            lengths themselves as sum len * 2^-len, at most 5.5 bits), else 2.
 // ---------------------------------------------------------------------------------------------------
 constexpr int KVC_LUT_MAX_BITS = 10;
 constexpr int KVC_LUT_MAX_LONG = 256;
-constexpr int KVC_LUT_HEADER_WORDS = 4;
+constexpr int KVC_LUT_HEADER_WORDS = 8;
 constexpr int KVC_LUT_LONG_WORDS = 2 * KVC_LUT_MAX_LONG;
 constexpr int KVC_LUT_ENTRY_WORDS = 1 << KVC_LUT_MAX_BITS;
 constexpr int KVC_LUT_FENTRY_OFFSET = KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS + KVC_LUT_ENTRY_WORDS;
 constexpr int KVC_LUT_WORDS = KVC_LUT_FENTRY_OFFSET + KVC_LUT_ENTRY_WORDS;
-constexpr int KVC_LUT_BYTES = KVC_LUT_WORDS * 4;          // 10256
+constexpr int KVC_LUT_BYTES = KVC_LUT_WORDS * 4;          // 10272
 constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2, rounded up
 
 // ---------------------------------------------------------------------------------------------------
 // host helpers (kvc_host.hip)
 // ---------------------------------------------------------------------------------------------------
 int kvc_fail(int code, const char *fmt, ...);
+// Tuning knobs settable through kvc_set_option (or, before first use, KVCOMP_<NAME> in the environment).
+enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_COUNT };
+int kvc_option(KvcOption which);
 int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the
 // reference-signature entry points derive from the decode tree on every call.
@@ -106,6 +115,45 @@ __device__ __forceinline__ float kvc_wave_sum(float v)
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
+}
+
+// Wave-wide reductions through the VALU's data-parallel lane permutes instead of LDS round trips; every lane
+// of the wave must be active.  Steps: neighbours within quads, quads within a row of 16, then the last lane
+// of a row is broadcast to the following row(s); lane 63 ends up with the total, which is read back as a scalar.
+template <class Op>
+__device__ __forceinline__ uint32_t kvc_wave_reduce_dpp(uint32_t v, Op op)
+{
+    constexpr int QUAD_SWAP1 = 0xB1, QUAD_SWAP2 = 0x4E, ROW_ROR4 = 0x124, ROW_ROR8 = 0x128, ROW_BCAST15 = 0x142,
+                  ROW_BCAST31 = 0x143;
+    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, QUAD_SWAP1, 0xf, 0xf, false));
+    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, QUAD_SWAP2, 0xf, 0xf, false));
+    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_ROR4, 0xf, 0xf, false));
+    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_ROR8, 0xf, 0xf, false));
+    // rows that receive nothing keep `old` = their own value, so they must not be combined with it: the
+    // operation is applied only where the row mask selects
+    {
+        const uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_BCAST15, 0xa, 0xf, false);
+        const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        if ((lane >> 4) & 1) v = op(v, t);
+    }
+    {
+        const uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_BCAST31, 0xc, 0xf, false);
+        const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        if (lane >= 32) v = op(v, t);
+    }
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+__device__ __forceinline__ float kvc_wave_sum_dpp(float v)
+{
+    return __uint_as_float(kvc_wave_reduce_dpp(__float_as_uint(v), [](uint32_t a, uint32_t b) {
+        return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
+    }));
+}
+
+__device__ __forceinline__ uint32_t kvc_wave_max_dpp(uint32_t v)
+{
+    return kvc_wave_reduce_dpp(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
 }
 
 // inclusive prefix sum over the 64 lanes of a wave

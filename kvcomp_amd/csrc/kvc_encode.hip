@@ -31,7 +31,7 @@ struct KvcEncodeArgs {
     uint8_t *encoded;
     int64_t encoded_cap;
     uint32_t base_global_offset;
-    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload
+    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload, [3] largest lane stream
     uint32_t *idx_offset;      // {tiles, bytes}  (include/kernels.h:34-42)
 };
 
@@ -65,9 +65,9 @@ __device__ __forceinline__ void kvc_load_vector(const KvcEncodeArgs &a, int64_t 
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs a)
 {
     __shared__ uint8_t s_len[256];
-    __shared__ uint32_t s_err;
+    __shared__ uint32_t s_err, s_longest;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) s_err = 0;
+    if (tid == 0) { s_err = 0; s_longest = 0; }
     {
         uint32_t len = 0;
         if (tid < a.table_entries) len = reinterpret_cast<const uint32_t *>(a.table)[2 * tid + 1];
@@ -101,9 +101,17 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs 
             reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[1] = end > 0xffffu ? 0xffffu : end;
         }
         if (err) atomicOr(&s_err, err);
+        uint32_t longest = bytes;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const uint32_t o = (uint32_t)__shfl_xor((int)longest, off, 64);
+            longest = o > longest ? o : longest;
+        }
+        if (lane == 0) atomicMax(&s_longest, longest);
     }
     __syncthreads();
     if (tid == 0 && s_err) atomicOr(&a.status[1], s_err);
+    if (tid == 0) atomicMax(&a.status[3], s_longest);
 }
 
 __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
@@ -213,7 +221,7 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
                               const uint8_t *d_encode_table, int64_t encode_table_bytes, uint8_t *d_block_infos,
                               uint8_t *d_thread_infos, uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                               uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes,
-                              int64_t *h_max_tile_bytes, void *stream_)
+                              int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     int64_t sizes[4];
@@ -251,8 +259,8 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     hipLaunchKernelGGL(kvc_encode_scan_kernel, dim3(1), dim3(1024), 0, stream, a);
     hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     KVC_HIP(hipGetLastError());
-    uint32_t h_status[3] = {0, 0, 0};
-    KVC_HIP(hipMemcpyAsync(h_status, slot, 12, hipMemcpyDeviceToHost, stream));
+    uint32_t h_status[4] = {0, 0, 0, 0};
+    KVC_HIP(hipMemcpyAsync(h_status, slot, 16, hipMemcpyDeviceToHost, stream));
     KVC_HIP(hipStreamSynchronize(stream));   // the reference returns after cudaDeviceSynchronize (kernels.cu:957)
     if (h_status[1] & KVC_ENC_ERR_NO_CODE) return kvc_fail(-3, "a symbol has no code in the encode table");
     if (h_status[1] & KVC_ENC_ERR_TILE_TOO_BIG)
@@ -261,6 +269,7 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
         return kvc_fail(-3, "payload (%u bytes) does not fit the encoded_data buffer (%lld bytes)", h_status[0], (long long)encoded_cap);
     *h_total_bytes = h_status[0];
     if (h_max_tile_bytes) *h_max_tile_bytes = h_status[2];
+    if (h_max_stream_bytes) *h_max_stream_bytes = h_status[3];
     return 0;
 }
 
@@ -268,22 +277,22 @@ extern "C" int kvc_k_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_
                                     int64_t encode_table_bytes, uint8_t *d_block_infos, uint8_t *d_thread_infos,
                                     uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                                     uint32_t base_global_offset, int64_t head_num, int64_t head_dim,
-                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, void *stream)
+                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream)
 {
     (void)head_num;
     return kvc_entropy_encode(1, d_sym, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
                               d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
-                              h_max_tile_bytes, stream);
+                              h_max_tile_bytes, h_max_stream_bytes, stream);
 }
 
 extern "C" int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride, const uint8_t *d_encode_table,
                                     int64_t encode_table_bytes, uint8_t *d_block_infos, uint8_t *d_thread_infos,
                                     uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                                     uint32_t base_global_offset, int64_t head_num, int64_t head_dim,
-                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, void *stream)
+                                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream)
 {
     (void)head_num;
     return kvc_entropy_encode(0, d_sym, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
                               d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
-                              h_max_tile_bytes, stream);
+                              h_max_tile_bytes, h_max_stream_bytes, stream);
 }

@@ -13,16 +13,20 @@
 // reach the FMA through v_readlane.  REP query heads share one KV head (grouped-query attention): the tile
 // is decoded once and feeds REP accumulators.
 //
-// Inner loop (the "fast" path, codes no longer than the table index):
-//   window  32 stream bits, rotated so that the next `lbits` bits sit at bits [lbits+1 : 2] -- masking gives
-//           the byte offset of the table entry directly
-//   entry   fp32 bit pattern of the symbol with (32 - len) in the 5 lowest mantissa bits: it is the FMA
-//           operand as it stands, and as a shift count it rotates the window left by len (v_alignbit)
-//   refill  every 4 (or 8) symbols the window is re-read from the staged payload at the lane's bit position;
-//           the entries are summed so the low byte of the sum gives the bits consumed
-// A 32-bit window always suffices for 8 symbols of <= 4 bits or 4 symbols of <= 8 bits.  With longer codes
-// 4 symbols can, very rarely, need more than 32 bits: lanes note the largest consumption they saw, and if
-// any lane went over, the wave decodes that tile again on the slow path.
+// Inner loop (the "fast" path, codes no longer than the table index).  The payload is staged in LDS with
+// every 32-bit word bit-reversed, so stream bit k is bit (k & 31) of word k >> 5 and a window is a plain
+// right funnel shift:
+//   window  32 stream bits, least significant first, held two bits up: the next `lbits` bits sit at bits
+//           [lbits+1 : 2], so masking gives the byte offset of the table entry directly
+//   entry   fp32 bit pattern of the symbol with the code length in its lowest mantissa byte: it is the FMA
+//           operand as it stands, and as a shift count it rotates the window right by len (v_alignbit)
+//   refill  every 4 (or 8) symbols the window is re-read from the staged payload at the lane's bit position
+//           (one ds_read2_b32 + one v_alignbit); the entries are summed, and the low byte of the sum is the
+//           number of bits consumed
+// A 32-bit window always suffices for 8 symbols of <= 4 bits or 4 symbols of <= 8 bits (two of the 32 bits
+// are the look-behind pair, hence 30 usable).  With longer codes 4 symbols can, very rarely, need more:
+// lanes note the largest consumption they saw, and if any lane went over, the wave decodes that tile again
+// on the slow path.
 //
 // Slow path (codebooks with codes longer than the table index, tiles larger than the staging area, or
 // the rare overflow above): one symbol per refill, generic table read from global memory, payload read
@@ -39,58 +43,44 @@ struct KvcFusedArgs {
     int out_f32;         // 0: fp16 (reference layout), 1: fp32
     int64_t tokens;
     int batch, kv_heads, q_heads, head_dim;
-    int stage_words;     // LDS words per wave for the staged payload
+    int table_words;     // LDS words reserved for the fused table (>= 1 << lbits of every codebook used)
+    int pack_words;      // LDS words per wave for the packed tile payload (multiple of 4, lead words included)
+    int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
 };
 
-constexpr int KVC_STAGE_LEAD_WORDS = 4;   // the payload is staged from word 4 on, so bit positions are never 0
+constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
+constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
 
-// -- staging ----------------------------------------------------------------------------------------
-struct KvcTile {
-    const uint32_t *gwords;   // 16-byte aligned global address of the chunk that holds the first payload byte
-    uint32_t nwords;          // whole words from gwords that contain payload bytes
-    uint32_t pos;             // this lane's first stream bit, counted from gwords (global) / from the stage base + lead
-    bool fits;                // payload is in LDS
+// What a tile needs from global memory, fetched into registers one tile ahead of its use.
+template <int REP, int SLOTS>
+struct KvcRaw {
+    uint4 pay[KVC_PRE_CHUNKS];        // payload chunks lane, lane + 64, ...
+    uint32_t off, bn;                 // block_info, clamped to the payload buffer (wave-uniform)
+    uint16_t ti_prev, ti_cur;         // thread_info of the previous lane (unused by lane 0) and of this lane
+    // operands of elements 2 * lane and 2 * lane + 1 (K: channels, V: tokens of the 128-token group), as loaded:
+    uint16_t sc[SLOTS][2];            // quantization scale (fp16 bits)
+    int8_t mn[SLOTS][2];              // quantization minimum
+    uint32_t x[SLOTS][REP];           // q / p (two fp16), per query head
 };
+// Nothing in it is touched before the tile is staged: any arithmetic on a loaded value would make the wave
+// wait for the load at that point and the fetch would no longer overlap the decode of the previous tile.
 
-__device__ __forceinline__ KvcTile kvc_stage_tile_lds(const KvcStreamArgs &a, int64_t tile, uint32_t *stage,
-                                                      int stage_words, int lane)
+// LDS traffic between the lanes of one wave needs no barrier (a wave's LDS operations complete in order);
+// this only keeps the compiler from moving accesses across the hand-over.
+__device__ __forceinline__ void kvc_wave_sync()
 {
-    const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile);
-    uint32_t off = bi[0];
-    uint32_t bn = bi[1] & 0xffffu;
-    if (bn > (uint32_t)KVC_MAX_TILE_BYTES) bn = KVC_MAX_TILE_BYTES;
-    if ((int64_t)off >= a.enc_bytes) bn = 0;
-    else if ((int64_t)off + bn > a.enc_bytes) bn = (uint32_t)(a.enc_bytes - off);
-    const uintptr_t src = reinterpret_cast<uintptr_t>(a.enc) + off;
-    const uintptr_t base = src & ~(uintptr_t)15;
-    const uint32_t head = (uint32_t)(src - base);
-    const uint32_t nchunks = bn ? (head + bn + 15u) >> 4 : 0u;
-    KvcTile t;
-    t.gwords = reinterpret_cast<const uint32_t *>(base);
-    t.nwords = (head + bn + 3u) >> 2;
-    // lead words + chunks + two look-ahead words must fit
-    t.fits = (int)(KVC_STAGE_LEAD_WORDS + 4 * nchunks + 2) <= stage_words;
-    if (t.fits) {
-        const uint4 *g = reinterpret_cast<const uint4 *>(base);
-        uint4 *s = reinterpret_cast<uint4 *>(stage + KVC_STAGE_LEAD_WORDS);
-        for (uint32_t c = lane; c < nchunks; c += KVC_WAVE) {
-            uint4 v = g[c];
-            v.x = kvc_bswap(v.x);
-            v.y = kvc_bswap(v.y);
-            v.z = kvc_bswap(v.z);
-            v.w = kvc_bswap(v.w);
-            s[c] = v;
-        }
-    }
-    uint32_t start = lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
-    if (start > bn) start = bn;
-    t.pos = (head + start) * 8u;
-    return t;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// memory byte j of a word carries stream bits 8j .. 8j+7, most significant first: a byte swap followed by a
+// full bit reversal leaves stream bit k of the word at bit k
+__device__ __forceinline__ uint32_t kvc_stream_word(uint32_t raw) { return __brev(kvc_bswap(raw)); }
+
 // -- slow path ----------------------------------------------------------------------------------------
-// One symbol per refill; table and long-code list in global memory; words from LDS (already big-endian)
-// or from global memory (raw, swapped on the fly, bounds-checked word by word).
+// One symbol per refill; table and long-code list in global memory; words from LDS (staged, bit-reversed)
+// or from global memory (raw, bounds-checked word by word).
 // Returns sum_i sym_i * ops[i * REP + r] for each query head r (ops: this lane's operand table in LDS).
 template <int REP>
 struct KvcVec {
@@ -110,8 +100,9 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
     for (int i = 0; i < n; i++) {
         const uint32_t wi = pos >> 5;
         uint32_t w0 = 0, w1 = 0;
-        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : words[wi];
-        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : words[wi + 1];
+        // either way the first stream bit of a word ends up in the most significant bit
+        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : __brev(words[wi]);
+        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : __brev(words[wi + 1]);
         const uint32_t hi = (uint32_t)(((((uint64_t)w0) << 32 | w1) << (pos & 31u)) >> 32);
         const uint32_t e = entries[hi >> lshift];
         uint32_t len = e & 0xffu, sym = (e >> 8) & 0xffu;
@@ -137,198 +128,388 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
 }
 
 // -- fast path ----------------------------------------------------------------------------------------
-// n symbols (a multiple of G) starting at bit t + 1 of the staged words; acc[r] += sym_i * ops[i * REP + r].
+// n symbols (a multiple of G) from bit u + 2 of the staged words on; acc[r] += sym_i * ops[i * REP + r].
 // `ops` is this lane's view of the wave's operand table in LDS: the same address in every lane (a broadcast
 // read) except in V tiles that straddle two heads, where the lanes of the second head point at its table.
-// Returns through `t` the new position and through `worst` the largest number of bits a group consumed.
+// Returns through `u` the new position and through `worst` the largest number of bits a group consumed.
+
+// LDS accessed by its byte offset: the table's offset is a multiple of its size, so "window bits | offset"
+// is the entry's address.
+typedef __attribute__((address_space(3))) uint32_t kvc_lds_u32;
+
 template <int G, bool CHECK, int REP>
-__device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t last_word, uint32_t &t,
-                                             const char *fentry_bytes, uint32_t mask4, uint32_t rot, int n,
+__device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t last_word, uint32_t &u,
+                                             uint32_t fentry_base, uint32_t mask4, int n,
                                              const float *ops, float (&acc)[REP], uint32_t &worst)
 {
 #pragma unroll 2
     for (int i = 0; i < n; i += G) {
-        uint32_t a = t >> 5;
+        uint32_t a = u >> 5;
         a = a < last_word ? a : last_word;
         const uint32_t w0 = stage[a], w1 = stage[a + 1];
         float op[G * REP];
+        if (G * REP >= 4) {
 #pragma unroll
-        for (int k = 0; k < G * REP; k += 4) {
-            const float4 v = *reinterpret_cast<const float4 *>(ops + i * REP + k);
-            op[k] = v.x;
-            if (k + 1 < G * REP) op[k + 1] = v.y;
-            if (k + 2 < G * REP) op[k + 2] = v.z;
-            if (k + 3 < G * REP) op[k + 3] = v.w;
+            for (int k = 0; k < G * REP; k += 4) {
+                const float4 v = *reinterpret_cast<const float4 *>(ops + i * REP + k);
+                op[k] = v.x;
+                op[k + 1] = v.y;
+                op[k + 2] = v.z;
+                op[k + 3] = v.w;
+            }
+        } else {   // G = 2, REP = 1
+            const float2 v = *reinterpret_cast<const float2 *>(ops + i * REP);
+            op[0] = v.x;
+            op[1] = v.y;
         }
-        const uint32_t win = __builtin_amdgcn_alignbit(w0, w1, ~t);   // 32 bits from stream bit t + 1
-        uint32_t R = __builtin_amdgcn_alignbit(win, win, rot);        // next lbits bits -> [lbits+1 : 2]
+        // 32 stream bits from bit u on: bits [1:0] are the pair before the lane's position, the next code
+        // starts at bit 2
+        uint32_t R = __builtin_amdgcn_alignbit(w1, w0, u);
         uint32_t es = 0;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            const uint32_t e = *reinterpret_cast<const uint32_t *>(fentry_bytes + (R & mask4));
-            R = __builtin_amdgcn_alignbit(R, R, e);                   // rotate left by len
+            const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
+            R = __builtin_amdgcn_alignbit(R, R, e);                   // rotate right by len
             es += e;
             const float f = __uint_as_float(e);
 #pragma unroll
             for (int r = 0; r < REP; r++) acc[r] = fmaf(f, op[g * REP + r], acc[r]);
         }
-        const uint32_t used = 32u * G - (es & 0xffu);
+        const uint32_t used = es & 0xffu;
         if (CHECK) worst = used > worst ? used : worst;
-        t += used;
+        u += used;
     }
 }
 
-// Operand table of one wave: [head slot (1 or 2)][128 elements][REP] floats.
-template <int REP>
-__host__ __device__ constexpr int kvc_op_words(int slots) { return slots * 128 * REP; }
+// -- tile geometry ------------------------------------------------------------------------------------
+// KIND 0: K tile (64 tokens x head_dim channels of one (batch, head); lane = token)
+// KIND 1: V tile (128 tokens x 64 flat channels; lane = channel), head_dim a multiple of 64: one head per tile
+// KIND 2: V tile with any other head_dim: the 64 channels may straddle two heads (two operand tables)
+template <int KIND>
+struct KvcGeom {
+    static constexpr bool IS_K = KIND == 0;
+    static constexpr int SLOTS = KIND == 2 ? 2 : 1;
+};
 
-template <int REP, bool IS_K>
-__global__ void __launch_bounds__(KVC_WG) kvc_fused_kernel(KvcFusedArgs a)
+// Issue the global loads of tile (row, col).  bi_off / bi_bn: the tile's block_info words.
+template <int REP, int KIND>
+__device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
+                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS> &raw)
 {
-    __shared__ __align__(16) uint32_t s_fentry[KVC_LUT_ENTRY_WORDS];   // static: its LDS offset folds into ds_read
-    extern __shared__ __align__(16) uint32_t smem[];                   // per wave: operand table, then staged payload
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    const int64_t tile = (int64_t)row * a.s.cols + col;
     const int D = a.head_dim;
-    const int slots = (!IS_K && (D % KVC_WAVE) != 0) ? 2 : 1;          // V tiles may straddle two heads
-    const int per_wave = kvc_op_words<REP>(slots) + a.stage_words;
-    float *ops = reinterpret_cast<float *>(smem + wave * per_wave);
-    uint32_t *stage = smem + wave * per_wave + kvc_op_words<REP>(slots);
+    // sizes are clamped so that corrupt metadata yields wrong symbols, never an out-of-bounds access
+    uint32_t off = bi_off, bn = bi_bn & 0xffffu;
+    if (bn > (uint32_t)KVC_MAX_TILE_BYTES) bn = KVC_MAX_TILE_BYTES;
+    if ((int64_t)off >= a.s.enc_bytes) bn = 0;
+    else if ((int64_t)off + bn > a.s.enc_bytes) bn = (uint32_t)(a.s.enc_bytes - off);
+    raw.off = off;
+    raw.bn = bn;
+    const int64_t ti0 = tile * KVC_WAVE + lane;
+    raw.ti_prev = a.s.thread_infos[ti0 > 0 ? ti0 - 1 : 0];
+    raw.ti_cur = a.s.thread_infos[ti0];
+    // payload: whole aligned 16-byte chunks that each hold at least one payload byte (such reads never leave
+    // the pages the payload lives in)
+    const uint8_t *src = a.s.enc + off;
+    const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
+    const uint32_t nchunks = bn ? (head + bn + 15u) >> 4 : 0u;
+    const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
+#pragma unroll
+    for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
+        const uint32_t c = lane + 64 * j;
+        if (c < nchunks) raw.pay[j] = g[c];
+    }
+    // operands; lanes past the end of a short vector load the last pair (ignored when staged)
+    const uint16_t *scale16 = reinterpret_cast<const uint16_t *>(a.scale);
+    if (KIND == 0) {
+        const int b = col / a.kv_heads, h = col - b * a.kv_heads;
+        const int e0 = 2 * lane < D ? 2 * lane : D - 2;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            // per-channel pairs, or one pair per 64-token block (kernels.cu:771-772)
+            const int64_t g = a.quant_mask == KVC_MASK_CHANNEL ? tile * D + e0 + half : (int64_t)row;
+            raw.sc[0][half] = scale16[g];
+            raw.mn[0][half] = a.min_i8[g];
+        }
+#pragma unroll
+        for (int r = 0; r < REP; r++)
+            raw.x[0][r] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
+    } else {
+        const int bh0 = (col * KVC_WAVE) / D;
+        const int bh_max = a.batch * a.kv_heads - 1;
+        const int64_t tk = (int64_t)row * KVC_V_TOKENS + 2 * lane;
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            int bh = bh0 + s;
+            bh = bh < bh_max ? bh : bh_max;                    // slot 1 is unused by a tile that ends the row
+            const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                int64_t g;
+                if (a.quant_mask == KVC_MASK_V_TOKEN) g = tk + half;
+                else if (a.quant_mask == KVC_MASK_SIM_TOKEN) g = (tk + half) * a.batch + b;
+                else g = ((tk + half) * a.batch + b) * a.kv_heads + h;           // KVC_MASK_VECTOR
+                raw.sc[s][half] = scale16[g];
+                raw.mn[s][half] = a.min_i8[g];
+            }
+#pragma unroll
+            for (int r = 0; r < REP; r++)
+                raw.x[s][r] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * a.tokens + tk);
+        }
+    }
+}
+
+__device__ __forceinline__ float kvc_half_bits_to_float(uint32_t bits16)
+{
+    return __half2float(__ushort_as_half((unsigned short)bits16));
+}
+
+// What the decode step needs to know about a staged tile.
+struct KvcStaged {
+    bool fits;            // staged in LDS (wave-uniform); otherwise decode from global memory
+    uint32_t u0;          // fast-path start position (two bits before the first code) in the lane's LDS words
+    const uint32_t *gwords;   // the lane's stream in global memory, from the aligned word holding its first byte
+    uint32_t gnwords, gpos;
+};
+
+// Move a fetched tile into LDS: payload -> packed area (-> per-lane rows), operands -> table; returns the
+// constant terms sum_i min_i * operand_i in bias[].
+template <int REP, int KIND>
+__device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int row, int col, int lane,
+                                                    const KvcRaw<REP, KvcGeom<KIND>::SLOTS> &raw, float *ops,
+                                                    uint32_t *pack, uint32_t *rows, float (&bias)[REP], int &sel_out)
+{
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    const int D = a.head_dim;
+    KvcStaged st;
+    // ---- payload
+    const uint32_t bn = raw.bn;
+    uint32_t start = lane ? (uint32_t)(raw.ti_prev >> 3) : 0u, end = (uint32_t)(raw.ti_cur >> 3);
+    if (start > bn) start = bn;
+    if (end > bn) end = bn;
+    if (end < start) end = start;
+    const uint8_t *src = a.s.enc + raw.off;
+    const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
+    const uint32_t nchunks = bn ? (head + bn + 15u) >> 4 : 0u;
+    const uint32_t first = head + start;                                   // byte offset in the packed area
+    const uint32_t nwords = end > start ? ((first & 3u) + (end - start) + 3u) >> 2 : 0u;
+    {
+        const uint8_t *lsrc = src + start;
+        const uint32_t skew = (uint32_t)(reinterpret_cast<uintptr_t>(lsrc) & 3u);
+        st.gwords = reinterpret_cast<const uint32_t *>(lsrc - skew);
+        st.gnwords = nwords;
+        st.gpos = skew * 8u;
+    }
+    // the packed area keeps row_words spare words at its end: the copy into rows below moves the same
+    // number of words for every lane, so the last lanes read past the payload
+    bool fits = KVC_PACK_LEAD + 4u * nchunks + 2u + (uint32_t)a.row_words <= (uint32_t)a.pack_words;
+    uint32_t longest = 0;
+    if (a.row_words) {
+        longest = kvc_wave_max_dpp(nwords);
+        fits = fits && longest + 2u <= (uint32_t)a.row_words;
+    }
+    st.fits = fits;
+    if (fits) {
+        uint4 *p4 = reinterpret_cast<uint4 *>(pack + KVC_PACK_LEAD);
+#pragma unroll
+        for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
+            const uint32_t c = lane + 64 * j;
+            if (c < nchunks) {
+                uint4 v = raw.pay[j];
+                v.x = kvc_stream_word(v.x);
+                v.y = kvc_stream_word(v.y);
+                v.z = kvc_stream_word(v.z);
+                v.w = kvc_stream_word(v.w);
+                p4[c] = v;
+            }
+        }
+        const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
+        for (uint32_t c = lane + 64 * KVC_PRE_CHUNKS; c < nchunks; c += KVC_WAVE) {   // tiles beyond 4 KiB
+            uint4 v = g[c];
+            v.x = kvc_stream_word(v.x);
+            v.y = kvc_stream_word(v.y);
+            v.z = kvc_stream_word(v.z);
+            v.w = kvc_stream_word(v.w);
+            p4[c] = v;
+        }
+    }
+    // ---- operand table: element i of head slot s, query head r at ops[(s * 128 + i) * REP + r]
+    float bias_s[SLOTS][REP];
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+#pragma unroll
+        for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f;
+        const bool live = KIND != 0 || 2 * lane < D;
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            const int i = 2 * lane + half;
+            const float sc = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
+            const float mn = (float)raw.mn[s][half];
+#pragma unroll
+            for (int r = 0; r < REP; r++) {
+                const float v = sc * kvc_half_bits_to_float((raw.x[s][r] >> (16 * half)) & 0xffffu);
+                ops[(s * 128 + i) * REP + r] = v;
+                bias_s[s][r] += mn * v;
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < REP; r++) bias_s[s][r] = kvc_wave_sum_dpp(bias_s[s][r]);
+    }
+    int sel = 0;
+    if (KIND == 2) {
+        const int c0 = col * KVC_WAVE;
+        sel = (c0 % D + lane) >= D;                                        // 1 past a head boundary
+    }
+    sel_out = sel;
+#pragma unroll
+    for (int r = 0; r < REP; r++) bias[r] = (SLOTS == 2 && sel) ? bias_s[SLOTS - 1][r] : bias_s[0][r];
+    kvc_wave_sync();
+    // ---- per-lane rows: [lead word][the words of the packed area that hold this lane's stream]
+    // Rows are an odd number of words apart, so lanes that are equally deep into their streams read 64
+    // different addresses spread evenly over the banks; in the packed area such lanes sit one stream length
+    // apart, which lines them up on a few banks whenever that length is close to a divisor of the bank count.
+    if (fits) {
+        const uint32_t w0 = KVC_PACK_LEAD + (first >> 2);
+        if (a.row_words) {
+            uint32_t *my_row = rows + lane * a.row_words + 1;
+            const uint32_t *my_pack = pack + w0;
+            // the same (even) number of words for every lane; what a lane copies beyond its own stream is
+            // never decoded.  Rows hold an even number of words after the lead word.
+            for (uint32_t k = 0; k < longest; k += 2) {
+                const uint32_t wa = my_pack[k], wb = my_pack[k + 1];
+                my_row[k] = wa;
+                my_row[k + 1] = wb;
+            }
+            st.u0 = 32u + (first & 3u) * 8u - 2u;
+            kvc_wave_sync();
+        } else {
+            st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;
+        }
+    } else {
+        st.u0 = 0;
+    }
+    return st;
+}
+
+template <int REP, int KIND>
+__global__ void __launch_bounds__(KVC_WG, REP == 1 ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
+{
+    constexpr bool IS_K = KIND == 0;
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    // dynamic LDS: the fused table (at offset 0, so that its address folds into the lookups), then per wave:
+    // operand table, packed payload, rows
+    extern __shared__ __align__(16) uint32_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int D = a.head_dim;
+    const int per_wave = SLOTS * 128 * REP + a.pack_words + KVC_WAVE * a.row_words;
+    uint32_t *s_fentry = smem;
+    float *ops = reinterpret_cast<float *>(smem + a.table_words + wave * per_wave);
+    uint32_t *pack = smem + a.table_words + wave * per_wave + SLOTS * 128 * REP;
+    uint32_t *rows = pack + a.pack_words;
     const int row = blockIdx.y;
     const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
     const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
-    const uint32_t lbits = lut_g[0], lmax = lut_g[1], nlong = lut_g[2];
-    const bool fast_book = nlong == 0 && lbits <= (uint32_t)KVC_LUT_MAX_BITS;
+    const uint32_t lbits = lut_g[0], nlong = lut_g[2];
+    const bool fast_book = nlong == 0 && (1u << lbits) <= (uint32_t)a.table_words;
     if (fast_book)
         for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) s_fentry[i] = lut_g[KVC_LUT_FENTRY_OFFSET + i];
-    if (lane < KVC_STAGE_LEAD_WORDS) stage[lane] = 0;
+    if (lane < KVC_PACK_LEAD) pack[lane] = 0;
+    if (a.row_words) rows[lane * a.row_words] = 0;
     __syncthreads();
     const uint32_t mask4 = ((1u << lbits) - 1u) << 2;
-    const uint32_t rot = 30u - lbits;                                  // (32 - lbits) - 2
-    const uint32_t last_word = (uint32_t)a.stage_words - 2u;
+    const uint32_t fgroup = lut_g[4], fcheck = lut_g[5];
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
+    const uint32_t fe = (uint32_t)(uintptr_t)(kvc_lds_u32 *)s_fentry;  // 0: the table opens the dynamic LDS
 
-    for (int it = 0; it < a.s.tiles_per_wave; it++) {
-        const int col = (blockIdx.x * KVC_WAVES_PER_WG + wave) * a.s.tiles_per_wave + it;
-        const bool active = col < a.s.cols;
-        const int64_t tile = (int64_t)row * a.s.cols + col;
-        KvcTile tl;
-        tl.fits = false;
-        float bias[REP];
-        int64_t out_base = 0, out_step = 0;
-        const float *my_ops = ops;
-        if (active) {
-            tl = kvc_stage_tile_lds(a.s, tile, stage, a.stage_words, lane);
-            // ---- per-tile operand table: element i of head slot s, query head r at ops[(s*128 + i)*REP + r]
-            if (IS_K) {
-                const int b = col / a.kv_heads, h = col - b * a.kv_heads;
+    // this wave's tiles: T consecutive columns of one tile row
+    const int T = a.s.tiles_per_wave;
+    const int col0 = (blockIdx.x * KVC_WAVES_PER_WG + wave) * T;
+    int ntiles = a.s.cols - col0;
+    ntiles = ntiles < T ? ntiles : T;
+    if (ntiles <= 0) return;
+    // block_info of tile col0 + j in lane j
+    uint32_t bi_off = 0, bi_bn = 0;
+    if (lane < ntiles) {
+        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.s.block_infos + 8 * ((int64_t)row * a.s.cols + col0 + lane));
+        bi_off = bi[0];
+        bi_bn = bi[1];
+    }
+    KvcRaw<REP, SLOTS> raw;
+    kvc_fetch_tile<REP, KIND>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    float bias[REP];
+    int sel = 0;
+    KvcStaged st = kvc_stage_tile<REP, KIND>(a, row, col0, lane, raw, ops, pack, rows, bias, sel);
+    for (int it = 0; it < ntiles; it++) {
+        const int col = col0 + it;
+        const bool more = it + 1 < ntiles;
+        if (more)   // loads for the next tile fly while this one is decoded
+            kvc_fetch_tile<REP, KIND>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
+                                      __builtin_amdgcn_readlane(bi_bn, it + 1), lane, raw);
+        const float *my_ops = ops + sel * 128 * REP;
+        float acc[REP];
 #pragma unroll
-                for (int r = 0; r < REP; r++) bias[r] = 0.f;
-#pragma unroll
-                for (int half = 0; half < 2; half++) {
-                    const int i = lane + 64 * half;
-                    float sc = 0.f, mn = 0.f;
-                    if (i < D) {
-                        if (a.quant_mask == KVC_MASK_CHANNEL) {
-                            sc = __half2float(a.scale[tile * D + i]);
-                            mn = (float)a.min_i8[tile * D + i];
-                        } else {   // KVC_MASK_K_BLOCK: one pair per 64-token block (kernels.cu:771-772)
-                            sc = __half2float(a.scale[row]);
-                            mn = (float)a.min_i8[row];
-                        }
-                    }
-#pragma unroll
-                    for (int r = 0; r < REP; r++) {
-                        const __half *qp = a.x + ((int64_t)b * a.q_heads + h * REP + r) * D;
-                        const float v = i < D ? sc * __half2float(qp[i]) : 0.f;
-                        ops[i * REP + r] = v;
-                        bias[r] += mn * v;
-                    }
-                }
-                out_base = ((int64_t)b * a.q_heads + h * REP) * a.tokens + (int64_t)row * KVC_WAVE + lane;
-                out_step = a.tokens;
+        for (int r = 0; r < REP; r++) acc[r] = 0.f;
+        bool redo = !(fast_book && st.fits);
+        if (!redo) {
+            const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
+            const uint32_t last_word = (uint32_t)(a.row_words ? a.row_words : a.pack_words) - 2u;
+            uint32_t u = st.u0, worst = 0;
+            if (fgroup >= 8 && !fcheck) {
+                kvc_fast_dot<8, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (fgroup >= 8) {
+                kvc_fast_dot<8, true, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (fgroup >= 4 && !fcheck) {
+                kvc_fast_dot<4, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (fgroup >= 4) {
+                kvc_fast_dot<4, true, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
             } else {
-                const int c0 = col * KVC_WAVE;                         // first flat channel of the tile
-                const int bh0 = c0 / D;
-                const int bh_lane = (c0 + lane) / D;
-                const int d = c0 + lane - bh_lane * D;
-                const int sel = bh_lane - bh0;                         // 0, or 1 past a head boundary
-                float bias_s[2][REP];
-#pragma unroll
-                for (int s = 0; s < 2; s++) {
-                    if (s < slots) {
-                        int bh = bh0 + s;
-                        const int bh_max = a.batch * a.kv_heads - 1;
-                        bh = bh < bh_max ? bh : bh_max;                // slot 1 is unused by a tile that ends the row
-                        const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
-#pragma unroll
-                        for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f;
-#pragma unroll
-                        for (int half = 0; half < 2; half++) {
-                            const int i = lane + 64 * half;
-                            const int64_t tk = (int64_t)row * KVC_V_TOKENS + i;
-                            int64_t g;
-                            if (a.quant_mask == KVC_MASK_V_TOKEN) g = tk;
-                            else if (a.quant_mask == KVC_MASK_SIM_TOKEN) g = tk * a.batch + b;
-                            else g = (tk * a.batch + b) * a.kv_heads + h;           // KVC_MASK_VECTOR
-                            const float sc = __half2float(a.scale[g]), mn = (float)a.min_i8[g];
-#pragma unroll
-                            for (int r = 0; r < REP; r++) {
-                                const __half *pp = a.x + ((int64_t)b * a.q_heads + h * REP + r) * a.tokens;
-                                const float v = sc * __half2float(pp[tk]);
-                                ops[(s * 128 + i) * REP + r] = v;
-                                bias_s[s][r] += mn * v;
-                            }
-                        }
-#pragma unroll
-                        for (int r = 0; r < REP; r++) bias_s[s][r] = kvc_wave_sum(bias_s[s][r]);
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < REP; r++) bias[r] = (slots == 2 && sel) ? bias_s[1][r] : bias_s[0][r];
-                my_ops = ops + sel * 128 * REP;
-                const int b = bh_lane / a.kv_heads, h = bh_lane - b * a.kv_heads;
-                out_base = (((int64_t)row * a.batch + b) * a.q_heads + h * REP) * D + d;
-                out_step = D;
+                kvc_fast_dot<2, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
             }
-            if (IS_K) {
-#pragma unroll
-                for (int r = 0; r < REP; r++) bias[r] = kvc_wave_sum(bias[r]);
-            }
+            redo = __any(worst > 30u);
         }
-        __syncthreads();
-        if (active) {
-            float acc[REP];
-#pragma unroll
-            for (int r = 0; r < REP; r++) acc[r] = 0.f;
-            bool redo = !(fast_book && tl.fits);
-            if (!redo) {
-                uint32_t t = tl.pos + 32u * KVC_STAGE_LEAD_WORDS - 1u, worst = 0;
-                const char *fe = reinterpret_cast<const char *>(s_fentry);
-                if (lmax <= 4) {
-                    kvc_fast_dot<8, false, REP>(stage, last_word, t, fe, mask4, rot, n, my_ops, acc, worst);
-                } else if (lmax <= 8) {
-                    kvc_fast_dot<4, false, REP>(stage, last_word, t, fe, mask4, rot, n, my_ops, acc, worst);
-                } else {
-                    kvc_fast_dot<4, true, REP>(stage, last_word, t, fe, mask4, rot, n, my_ops, acc, worst);
-                    redo = __any(worst > 32u);
-                }
-            }
-            if (redo) {
-                const KvcVec<REP> res = tl.fits
-                    ? kvc_slow_tile<REP, false>(stage, (uint32_t)a.stage_words, tl.pos + 32u * KVC_STAGE_LEAD_WORDS, lut_g, n, my_ops)
-                    : kvc_slow_tile<REP, true>(tl.gwords, tl.nwords, tl.pos, lut_g, n, my_ops);
-#pragma unroll
-                for (int r = 0; r < REP; r++) acc[r] = res.v[r];
+        if (redo) {
+            KvcVec<REP> res;
+            if (st.fits) {
+                const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
+                const uint32_t nw = (uint32_t)(a.row_words ? a.row_words : a.pack_words);
+                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + 2u, lut_g, n, my_ops);
+            } else {
+                res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops);
             }
 #pragma unroll
-            for (int r = 0; r < REP; r++) {
-                const int64_t o = out_base + r * out_step;
-                const float v = acc[r] + bias[r];
-                if (a.out_f32) reinterpret_cast<float *>(a.out)[o] = v;
-                else reinterpret_cast<__half *>(a.out)[o] = __float2half(v);
-            }
+            for (int r = 0; r < REP; r++) acc[r] = res.v[r];
         }
-        __syncthreads();
+        // ---- results
+        int64_t out_base, out_step;
+        if (IS_K) {
+            const int b = col / a.kv_heads, h = col - b * a.kv_heads;
+            out_base = ((int64_t)b * a.q_heads + h * REP) * a.tokens + (int64_t)row * KVC_WAVE + lane;
+            out_step = a.tokens;
+        } else {
+            const int c0 = col * KVC_WAVE;
+            const int bh0 = c0 / D, d0 = c0 - bh0 * D;                  // wave-uniform
+            const int past = (KIND == 2 && d0 + lane >= D) ? 1 : 0;     // this lane's channel lies in the next head
+            const int bh = bh0 + past, d = d0 + lane - past * D;
+            const int b0 = bh0 / a.kv_heads, h0 = bh0 - b0 * a.kv_heads;
+            const int wrap = (h0 + past == a.kv_heads) ? 1 : 0;         // ... which may be the first head of the next batch entry
+            const int b = b0 + wrap, h = wrap ? 0 : h0 + past;
+            (void)bh;
+            out_base = (((int64_t)row * a.batch + b) * a.q_heads + h * REP) * D + d;
+            out_step = D;
+        }
+#pragma unroll
+        for (int r = 0; r < REP; r++) {
+            const int64_t o = out_base + r * out_step;
+            const float v = acc[r] + bias[r];
+            if (a.out_f32) reinterpret_cast<float *>(a.out)[o] = v;
+            else reinterpret_cast<__half *>(a.out)[o] = __float2half(v);
+        }
+        if (more) {
+            kvc_wave_sync();     // every lane is done reading this tile's LDS data
+            st = kvc_stage_tile<REP, KIND>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel);
+        }
     }
 }
 
@@ -336,30 +517,66 @@ __global__ void __launch_bounds__(KVC_WG) kvc_fused_kernel(KvcFusedArgs a)
 // host side
 // ---------------------------------------------------------------------------------------------------
 template <int REP>
-static void kvc_launch_fused(int is_k, const KvcFusedArgs &a, dim3 grid, size_t lds, hipStream_t stream)
+static void kvc_launch_fused(int kind, const KvcFusedArgs &a, dim3 grid, size_t lds, hipStream_t stream)
 {
-    if (is_k) hipLaunchKernelGGL((kvc_fused_kernel<REP, true>), grid, dim3(KVC_WG), lds, stream, a);
-    else hipLaunchKernelGGL((kvc_fused_kernel<REP, false>), grid, dim3(KVC_WG), lds, stream, a);
+    if (kind == 0) hipLaunchKernelGGL((kvc_fused_kernel<REP, 0>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 1) hipLaunchKernelGGL((kvc_fused_kernel<REP, 1>), grid, dim3(KVC_WG), lds, stream, a);
+    else hipLaunchKernelGGL((kvc_fused_kernel<REP, 2>), grid, dim3(KVC_WG), lds, stream, a);
 }
 
-// LDS words per wave for the staged payload: room for about twice the average tile (tiles that still do
-// not fit are decoded from global memory), between 1 KiB and the largest tile the format allows.
-static int kvc_pick_stage_words(int64_t encoded_bytes, int64_t tiles, int64_t max_tile_bytes)
+// LDS layout of one workgroup: the fused table, then per wave the operand table(s), the packed payload of
+// one tile and (optionally) the per-lane rows.  Sized from the encoder's hints (largest tile payload,
+// longest lane stream); without them from twice the payload's means.  Tiles that do not fit are decoded
+// from global memory, so the sizes only affect speed.  Everything stays within 64 KiB per workgroup.
+static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_bytes, int64_t tiles,
+                           int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits)
 {
-    static int forced = -1;
-    if (forced < 0) {
-        const char *e = std::getenv("KVC_STAGE_BYTES");
-        forced = e ? std::atoi(e) : 0;
+    const int force_rows = kvc_option(KVC_OPT_FUSED_ROWS);   // 0 / 1 overrides the choice below
+    a.table_words = 1 << ((max_code_bits >= 1 && max_code_bits <= KVC_LUT_MAX_BITS) ? max_code_bits : KVC_LUT_MAX_BITS);
+    if (a.table_words < 4) a.table_words = 4;   // keeps the per-wave areas 16-byte aligned
+    const int64_t ops_words = (int64_t)slots * 128 * rep;
+    const int64_t budget = (65536 / 4 - a.table_words) / KVC_WAVES_PER_WG - ops_words;   // words per wave
+    const int64_t mean_tile = encoded_bytes / (tiles > 0 ? tiles : 1);
+    int64_t tile_bytes = max_tile_bytes > 0 ? max_tile_bytes : 2 * mean_tile + 64;
+    if (tile_bytes > KVC_MAX_TILE_BYTES) tile_bytes = KVC_MAX_TILE_BYTES;
+    // lead words + the payload's chunks (it may start anywhere in its first chunk) + look-ahead
+    int64_t pack = KVC_PACK_LEAD + ((tile_bytes + 15 + 15) / 16) * 4 + 4;
+    int64_t stream_bytes = max_stream_bytes > 0 ? max_stream_bytes : 2 * mean_tile / KVC_WAVE + 4;
+    // lead word + the stream's words (it may start anywhere in its first word) + look-ahead, forced odd
+    const int64_t row = ((stream_bytes + 3 + 3) / 4 + 2) | 1;
+    const int64_t pack_rows = (pack + row + 3) / 4 * 4;      // spare words for the fixed-length copy into rows
+    // Rows cost LDS space and a copy; they pay when decoding from the packed payload would line the lanes up
+    // on a few banks: lane l reads about l mean-stream-lengths into the payload, so if a small multiple of
+    // that length is close to a multiple of the 32 banks, every k-th lane hits the same bank.
+    const double mean_stream_words = (double)encoded_bytes / (double)(tiles > 0 ? tiles : 1) / KVC_WAVE / 4.0;
+    bool use_rows = false;
+    for (int k = 1; k <= 4; k++) {
+        const double x = k * mean_stream_words / 32.0;
+        const double dist = (x - (double)(int64_t)(x + 0.5)) * 32.0;
+        if (x >= 0.5 && dist > -1.0 && dist < 1.0) use_rows = true;
     }
-    // payload + up to 15 bytes before it in its first chunk, rounded up to chunks, + lead and look-ahead words
-    int64_t bytes = max_tile_bytes > 0 ? ((max_tile_bytes + 15 + 15) / 16) * 16 + 4 * (KVC_STAGE_LEAD_WORDS + 2)
-                                       : 2 * (encoded_bytes / (tiles > 0 ? tiles : 1)) + 64;
-    if (forced > 0) bytes = forced;
-    const int64_t max_bytes = ((KVC_MAX_TILE_BYTES + 15 + 15) / 16) * 16 + 16 * KVC_STAGE_LEAD_WORDS / 4 + 16;
-    if (bytes < 1024) bytes = 1024;
-    if (bytes > max_bytes) bytes = max_bytes;
-    bytes = (bytes + 255) / 256 * 256;
-    return (int)(bytes / 4);
+    if (force_rows >= 0) use_rows = force_rows != 0;
+    if (use_rows && pack_rows + KVC_WAVE * row <= budget) {
+        a.row_words = (int)row;
+        pack = pack_rows;
+    } else {
+        a.row_words = 0;
+    }
+    if (pack > budget) pack = budget / 4 * 4;
+    a.pack_words = (int)pack;
+    return 4 * ((size_t)a.table_words +
+                (size_t)KVC_WAVES_PER_WG * (size_t)(ops_words + a.pack_words + KVC_WAVE * a.row_words));
+}
+
+// Consecutive tiles of a row that one wave works through (fetching one ahead): as many as still leave
+// every SIMD of the chip several waves.
+static int kvc_plan_tiles_per_wave(int64_t tiles)
+{
+    const int forced = kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE);
+    if (forced > 0) return forced > 64 ? 64 : forced;
+    // measured on MI355X: two is best once there are enough tiles (the fetch of the second overlaps the
+    // decode of the first); longer runs only leave fewer workgroups to balance over the chip
+    return tiles >= 2 * 256 * 4 * 5 ? 2 : 1;
 }
 
 static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
@@ -368,7 +585,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                      const int8_t *d_min, const void *d_scale, int quant_mask, const void *d_x, void *d_out,
                      int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                      float *elapsed_ms, void *stream_, const uint32_t *d_luts = nullptr, int rows_per_codebook = 0,
-                     int out_f32 = 0, int64_t max_tile_bytes = 0)
+                     int out_f32 = 0, int64_t max_tile_bytes = 0, int64_t max_stream_bytes = 0, int max_code_bits = 0)
 {
     hipStream_t stream = (hipStream_t)stream_;
     if (tokens == 0) {
@@ -408,19 +625,20 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     a.kv_heads = (int)kv_heads;
     a.q_heads = (int)q_heads;
     a.head_dim = (int)head_dim;
-    a.stage_words = kvc_pick_stage_words(encoded_bytes, rows * a.s.cols, max_tile_bytes);
-    const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
-    const size_t lds = (size_t)KVC_WAVES_PER_WG * (size_t)(slots * 128 * rep + a.stage_words) * 4;   // operand tables + staging
+    const int kind = is_k ? 0 : (head_dim % KVC_WAVE == 0 ? 1 : 2);
+    const size_t lds = kvc_plan_lds(a, kind == 2 ? 2 : 1, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
+                                    max_stream_bytes, max_code_bits);
+    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
     KvcTimer timer(elapsed_ms, stream);
     if (!d_luts) {
         if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
     }
     const dim3 grid = kvc_grid(a.s, rows);
     switch (rep) {
-        case 1: kvc_launch_fused<1>(is_k, a, grid, lds, stream); break;
-        case 2: kvc_launch_fused<2>(is_k, a, grid, lds, stream); break;
-        case 4: kvc_launch_fused<4>(is_k, a, grid, lds, stream); break;
-        default: kvc_launch_fused<8>(is_k, a, grid, lds, stream); break;
+        case 1: kvc_launch_fused<1>(kind, a, grid, lds, stream); break;
+        case 2: kvc_launch_fused<2>(kind, a, grid, lds, stream); break;
+        case 4: kvc_launch_fused<4>(kind, a, grid, lds, stream); break;
+        default: kvc_launch_fused<8>(kind, a, grid, lds, stream); break;
     }
     KVC_HIP(hipGetLastError());
     return timer.finish();
@@ -472,26 +690,26 @@ extern "C" int kvc_k_scores_lut(const void *d_luts, int64_t rows_per_codebook, c
                                 int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                                 const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                                 const void *d_quant_scales_f16, int quant_mask, const void *d_q_f16, void *d_scores,
-                                int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
+                                int out_f32, int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t tokens, int64_t batch, int64_t kv_heads,
                                 int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream)
 {
     KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
     return kvc_fused(1, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
                      d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_q_f16, d_scores, tokens,
                      batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
-                     (int)rows_per_codebook, out_f32, max_tile_bytes);
+                     (int)rows_per_codebook, out_f32, max_tile_bytes, max_stream_bytes, max_code_bits);
 }
 
 extern "C" int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint8_t *d_block_infos,
                                   int64_t block_infos_bytes, const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
                                   const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_quant_min_ints,
                                   const void *d_quant_scales_f16, int quant_mask, const void *d_p_f16, void *d_partial,
-                                  int out_f32, int64_t max_tile_bytes, int64_t tokens, int64_t batch, int64_t kv_heads,
+                                  int out_f32, int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t tokens, int64_t batch, int64_t kv_heads,
                                   int64_t q_heads, int64_t head_dim, float *elapsed_ms, void *stream)
 {
     KVC_REQUIRE(d_luts != nullptr, "d_luts is NULL");
     return kvc_fused(0, nullptr, 0, KVC_TREE_I8, d_block_infos, block_infos_bytes, d_thread_infos, thread_infos_bytes,
                      d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_p_f16, d_partial, tokens,
                      batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
-                     (int)rows_per_codebook, out_f32, max_tile_bytes);
+                     (int)rows_per_codebook, out_f32, max_tile_bytes, max_stream_bytes, max_code_bits);
 }

@@ -2,7 +2,9 @@
 // buffer sizing and the host Huffman codebook builder.
 #include "kvc_common.h"
 
+#include <atomic>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -31,7 +33,50 @@ int kvc_check_hip(hipError_t e, const char *what)
 }
 
 extern "C" const char *kvc_last_error(void) { return g_last_error.c_str(); }
-extern "C" int kvc_abi_version(void) { return 1; }
+extern "C" int kvc_abi_version(void) { return 2; }
+
+// ---------------------------------------------------------------------------------------------------
+// tuning knobs
+// ---------------------------------------------------------------------------------------------------
+namespace {
+struct OptionDef {
+    const char *name;
+    const char *env;
+    int fallback;
+};
+const OptionDef g_option_defs[KVC_OPT_COUNT] = {
+    {"fused_rows", "KVCOMP_FUSED_ROWS", -1},                     // -1 choose per call, 0 never, 1 whenever it fits
+    {"fused_tiles_per_wave", "KVCOMP_FUSED_TILES_PER_WAVE", 0},  // 0 choose per call
+};
+std::atomic<int> g_options[KVC_OPT_COUNT];
+std::once_flag g_options_once;
+void init_options()
+{
+    for (int i = 0; i < KVC_OPT_COUNT; i++) {
+        const char *e = std::getenv(g_option_defs[i].env);
+        g_options[i].store(e ? std::atoi(e) : g_option_defs[i].fallback);
+    }
+}
+}  // namespace
+
+int kvc_option(KvcOption which)
+{
+    std::call_once(g_options_once, init_options);
+    return g_options[which].load(std::memory_order_relaxed);
+}
+
+extern "C" int kvc_set_option(const char *name, int value)
+{
+    KVC_REQUIRE(name != nullptr, "option name is NULL");
+    std::call_once(g_options_once, init_options);
+    for (int i = 0; i < KVC_OPT_COUNT; i++) {
+        if (std::strcmp(name, g_option_defs[i].name) == 0) {
+            g_options[i].store(value);
+            return 0;
+        }
+    }
+    return kvc_fail(-1, "unknown option '%s'", name);
+}
 
 // ---------------------------------------------------------------------------------------------------
 // per-device scratch ring: KVC_WS_SLOTS slots handed out round-robin.  A slot is reused after

@@ -19,6 +19,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
     __shared__ uint8_t s_leaf[KVC_TREE_MAX_NODES];
     __shared__ uint8_t s_bit[KVC_TREE_MAX_NODES];
     __shared__ uint32_t s_lmax, s_nlong;
+    __shared__ float s_avg;   // sum over leaves of len * 2^-len: the mean code length if the code is well matched
 
     const int tid = threadIdx.x;
     const uint8_t *tree = trees + (int64_t)blockIdx.x * tree_stride;
@@ -26,7 +27,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
     int n_nodes = tree_bytes / node_bytes;
     if (n_nodes > KVC_TREE_MAX_NODES) n_nodes = KVC_TREE_MAX_NODES;
 
-    if (tid == 0) { s_lmax = 0; s_nlong = 0; }
+    if (tid == 0) { s_lmax = 0; s_nlong = 0; s_avg = 0.f; }
     for (int n = tid; n < KVC_TREE_MAX_NODES; n += KVC_WG) {
         int leaf = 0, a = -1, b = -1;
         if (n < n_nodes) {
@@ -78,6 +79,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
                 my_len[k] = len;
                 my_code[k] = code;
                 atomicMax(&s_lmax, len);
+                atomicAdd(&s_avg, (float)len * exp2f(-(float)len));
             }
         }
     }
@@ -107,8 +109,19 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
             cur = s_child[(idx >> (lbits - 1 - depth)) & 1u][cur];
         }
         entries[idx] = e;
-        const uint32_t len = e & 0xffu, sym = e >> 8;
-        lut[KVC_LUT_FENTRY_OFFSET + idx] = len ? (__float_as_uint((float)sym) | ((32u - len) & 31u)) : 31u;
+    }
+    // fused-kernel entries: the index bits are the stream bits in arrival order from bit 0 up (the fused
+    // kernels keep their window least-significant-bit first), so walk with bit j of the index at depth j
+    for (uint32_t idx = tid; idx < (1u << lbits); idx += KVC_WG) {
+        uint32_t e = 1u;                       // no code / code longer than the index: "symbol 0, length 1"
+        int cur = (int)(idx & 1u);
+        for (uint32_t depth = 1; depth <= lbits; depth++) {
+            if (cur < 0 || cur >= n_nodes) break;
+            if (s_leaf[cur]) { e = __float_as_uint((float)(s_child[0][cur] & 0xff)) | depth; break; }
+            if (depth == lbits) break;
+            cur = s_child[(idx >> depth) & 1u][cur];
+        }
+        lut[KVC_LUT_FENTRY_OFFSET + idx] = e;
     }
     __syncthreads();
     if (tid == 0) {
@@ -118,6 +131,12 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
         lut[1] = lmax;
         lut[2] = nlong;
         lut[3] = group;
+        const bool roomy = s_avg <= 5.5f;
+        const bool roomy8 = lmax == 4 && s_avg <= 2.75f;
+        lut[4] = (lmax <= 3 || roomy8) ? 8u : lmax <= 7 ? 4u : roomy ? 4u : 2u;
+        lut[5] = (roomy8 || (lmax > 7 && roomy)) ? 1u : 0u;
+        lut[6] = 0;
+        lut[7] = 0;
     }
 }
 

@@ -10,7 +10,6 @@
 #pragma once
 #include "kvc_common.h"
 
-#include <cstdlib>
 
 struct KvcStreamArgs {
     const uint8_t *enc;            // concatenated tile payloads
@@ -130,18 +129,6 @@ __device__ __forceinline__ void kvc_dispatch_group(const uint32_t *s_lut, Body &
 // ---------------------------------------------------------------------------------------------------
 // host side: geometry checks and launch shape shared by the decoders
 // ---------------------------------------------------------------------------------------------------
-static inline int kvc_tiles_per_wave(int64_t tiles)
-{
-    static int forced = -1;
-    if (forced < 0) {
-        const char *e = std::getenv("KVC_TILES_PER_WAVE");
-        forced = e ? std::atoi(e) : 0;
-    }
-    if (forced > 0) return forced;
-    (void)tiles;
-    return 1;   // measured on MI355X: one tile per wave is fastest at every size (more tiles only add latency)
-}
-
 static inline int kvc_fill_stream_args(KvcStreamArgs &s, const uint8_t *d_encoded, int64_t encoded_bytes,
                                 const uint8_t *d_block_infos, int64_t block_infos_bytes,
                                 const uint8_t *d_thread_infos, int64_t thread_infos_bytes, const uint32_t *d_luts,
@@ -174,7 +161,7 @@ static inline int kvc_fill_stream_args(KvcStreamArgs &s, const uint8_t *d_encode
     s.luts = d_luts;
     s.rows_per_codebook = 0;
     s.cols = (int)cols;
-    s.tiles_per_wave = kvc_tiles_per_wave(rows * cols);
+    s.tiles_per_wave = 1;
     s.vec_len = is_k ? (int)head_dim : KVC_V_TOKENS;
     s.stride = stride;
     *rows_out = rows;

@@ -165,7 +165,9 @@ class KVCompCtx:
         self._min_ints = _Growable()
         self._scales = _Growable()
         self.buffer: Optional[torch.Tensor] = None
-        self.max_tile_bytes = 0          # largest tile payload seen so far (sizes the fused decoders' LDS staging)
+        self.max_code_bits = 0           # longest code of the codebook (0 = unknown)
+        self.max_tile_bytes = 0            # largest tile payload seen so far (sizes the fused decoders' LDS staging)
+        self.max_stream_bytes = 0          # longest lane stream seen so far (sizes the fused decoders' LDS rows)
         self.encode_codebook: Optional[torch.Tensor] = None
         self.decode_codebook: Optional[torch.Tensor] = None
 
@@ -210,12 +212,12 @@ class KVCompCtx:
         if self.encode_codebook is None:     # first stored chunk defines the codebook (kvcomp_encode.py:99-103)
             shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
             assert shift == 0, "shift must be 0"
-            self.encode_codebook = enc.to(self.device)
-            self.decode_codebook = dec.to(self.device)
+            self._set_codebook(enc, dec)
         fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
         encoded_, block_infos_, vec_infos_ = fn(quant_ints, self.encode_codebook, bi_buf, ti_buf, idx_buf, payload_buf,
                                                 self._encoded.used, self.head_num, self.head_dim)
         self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
+        self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
         self._encoded.append(encoded_)
         self._block_infos.append(block_infos_)
         self._thread_infos.append(vec_infos_)
@@ -304,6 +306,12 @@ class KVCompCtx:
         if self.device is None:
             self.device = device_
             KVCompCtx.buffer_ctx_len[self.device] = 0
+        self._set_codebook(enc, dec)
+
+    def _set_codebook(self, enc: torch.Tensor, dec: torch.Tensor):
+        """enc / dec: CPU byte tensors from kvcomp_cuda.build_codebook."""
+        lengths = enc.view(torch.int32)[1::2]
+        self.max_code_bits = int(lengths.max())      # sizes the fused decoders' table in LDS
         self.encode_codebook = enc.to(self.device)
         self.decode_codebook = dec.to(self.device)
 

@@ -31,7 +31,8 @@ V_VEC_LEN = 128
 V_VEC_PER_BLK = 64
 
 # largest tile payload of the most recent encode call (a sizing hint for the table-driven fused decoders)
-last_encode_max_tile_bytes = 0
+last_encode_max_tile_bytes = 0      # largest tile payload / longest lane stream of the latest encode call:
+last_encode_max_stream_bytes = 0    # sizing hints for the table-driven fused decoders
 
 MASK_K_BLOCK, MASK_V_TOKEN, MASK_CHANNEL, MASK_SIM_TOKEN, MASK_VECTOR, MASK_SIM_BLOCK = 0xF, 0xE, 0x1, 0xC, 0x8, 0xD
 TREE_I8, TREE_I16 = 3, 5
@@ -113,15 +114,16 @@ def _entropy_encode(is_k, input, encode_code_book, block_infos, thread_infos, id
     _require(block_infos.numel() >= sizes[0], "block_infos buffer too small")
     _require(thread_infos.numel() >= sizes[1], "thread_infos buffer too small")
     _require(idx_offset.numel() >= sizes[2], "idx_offset buffer too small")
-    total, max_tile = C.c_int64(0), C.c_int64(0)
+    total, max_tile, max_stream = C.c_int64(0), C.c_int64(0), C.c_int64(0)
     fn = _lib.lib().kvc_k_entropy_encode if is_k else _lib.lib().kvc_v_entropy_encode
     with torch.cuda.device(input.device):
         check(fn(_ptr(input), tokens, stride, _ptr(encode_code_book), encode_code_book.numel(), _ptr(block_infos),
                  _ptr(thread_infos), _ptr(idx_offset), _ptr(encoded_data), encoded_data.numel(),
-                 int(base_global_offset) & 0xFFFFFFFF, head_num, head_dim, C.byref(total), C.byref(max_tile),
+                 int(base_global_offset) & 0xFFFFFFFF, head_num, head_dim, C.byref(total), C.byref(max_tile), C.byref(max_stream),
                  _stream(input)))
-    global last_encode_max_tile_bytes
+    global last_encode_max_tile_bytes, last_encode_max_stream_bytes
     last_encode_max_tile_bytes = int(max_tile.value)
+    last_encode_max_stream_bytes = int(max_stream.value)
     return encoded_data[:total.value], block_infos[:sizes[0]], thread_infos[:sizes[1]]
 
 

@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(raw, n), "libkvcomp_hip.so does not export %s" % n
     assert sorted(_lib.EXPORTED_SYMBOLS) == names          # the Python binding covers the whole header
-    assert _lib.lib().kvc_abi_version() == 1
+    assert _lib.lib().kvc_abi_version() == 2
 
 
 def test_missing_library_fails_loudly(monkeypatch):

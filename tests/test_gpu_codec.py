@@ -327,3 +327,33 @@ def test_fused_with_long_codes_uses_slow_path(is_k, nsym):
         m.v_decode_and_mat_vec_mul_cuda_export(*args, p.to(DEV), part, H, D)
         got = part.float().sum(0).cpu().numpy()
     assert np.abs(got - ref).max() <= 1e-3 * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("nsym,expect_lmax", [(200, 8), (12, 4), (7, 3)])
+def test_fused_k_window_groupings(nsym, expect_lmax):
+    """Near-uniform alphabets pin the code length, hence which window grouping the fused kernel takes:
+    200 symbols -> 8-bit codes, too dense for four per window (two per refill); 12 -> 4-bit codes (four per
+    refill, guaranteed); 7 -> 3-bit codes (eight per refill).  The 200-symbol book needs the int16 tree."""
+    rng = np.random.default_rng(21)
+    m = kc()
+    T, B, H, D = 128, 1, 2, 64
+    sym = rng.integers(0, nsym, size=(T // 64, 64, B, H, D)).astype(np.uint8)
+    fmt = m.TREE_I16 if nsym > 64 else m.TREE_I8
+    shift, enc, dec = m.build_codebook([_dev(sym)], tree_format=fmt)
+    counts = np.bincount(sym.ravel(), minlength=256).astype(np.int64)
+    assert int(O.huffman_build(counts)[1].max()) == expect_lmax
+    sizes = m.calculate_buffer_size(_dev(sym), True, H, D)
+    bufs = [torch.zeros(n, dtype=torch.uint8, device=DEV) for n in sizes]
+    g_enc, g_bi, g_ti = m.k_entropy_encode_cuda_export(_dev(sym), enc.to(DEV), bufs[0], bufs[1], bufs[2], bufs[3], 0, H, D)
+    ref_payload, _, _ = O.encode_tiles(sym, True, enc.numpy(), 0, vec_len=D)
+    assert np.array_equal(g_enc.cpu().numpy(), ref_payload)
+    gs = O.group_shape(sym.shape, O.MASK_CHANNEL)
+    mn = rng.integers(-(nsym // 2) - 1, 0, size=gs).astype(np.int8)       # symbols centred on zero, like real groups
+    scale = rng.uniform(0.01, 0.2, size=gs).astype(np.float16)
+    q = S.synth_q(B, H, D)
+    ref = O.fused_k(sym.reshape(T, B, H, D), mn, scale, O.MASK_CHANNEL, 64, S.np16(q))
+    out = torch.zeros(B, H, T, dtype=torch.float16, device=DEV)
+    m.k_decode_and_mat_vec_mul_cuda_export(dec.to(DEV), g_bi, g_ti, g_enc, _dev(mn.ravel()),
+                                           _dev(scale.ravel().view(np.uint16), torch.float16), q.to(DEV), out, H, D,
+                                           tree_format=fmt)
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= 1e-3 * np.abs(ref).max()

@@ -162,3 +162,64 @@ def test_compressed_attention_matches_fp32_reference(k_mode, rep, extra):
     s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
     ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
     assert (out - ref).abs().max() <= 1e-3 * ref.abs().max()
+
+
+@pytest.mark.parametrize("rows", [0, 1])
+@pytest.mark.parametrize("tiles_per_wave", [1, 2, 3])
+@pytest.mark.parametrize("D", [128, 96])
+def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D):
+    """The fused kernels may decode from the packed payload or from per-lane rows, and a wave may take one
+    tile or a run of tiles (fetching one ahead): every combination must give the same attention output,
+    including runs that are cut short at the end of a tile row (3 does not divide the tile columns)."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant")
+    T, B, H, rep = 512 + 19, 2, 4, 2
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    assert 0 < kctx.max_stream_bytes <= kctx.max_tile_bytes and 0 < kctx.max_code_bits <= 32
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    L = _lib.lib()
+    default_plan = CompressedAttention(kctx, vctx).attend(q)
+    try:
+        assert L.kvc_set_option(b"fused_rows", rows) == 0
+        assert L.kvc_set_option(b"fused_tiles_per_wave", tiles_per_wave) == 0
+        out = CompressedAttention(kctx, vctx).attend(q)
+    finally:
+        L.kvc_set_option(b"fused_rows", -1)
+        L.kvc_set_option(b"fused_tiles_per_wave", 0)
+    kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+    s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
+    ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
+    # the plan changes where the bits are read from, not the arithmetic: results are identical
+    assert torch.equal(out, default_plan)
+    # get() rounds every dequantized element to fp16, the fused kernels do not: the softmax turns that into
+    # a few 1e-3 of the output here
+    assert (out - ref).abs().max() <= 3e-3 * ref.abs().max()
+    assert L.kvc_set_option(b"no_such_option", 1) != 0
+
+
+@pytest.mark.parametrize("hint", ["too_small", "absent"])
+def test_compressed_attention_with_wrong_or_missing_size_hints(hint):
+    """The encoder's size hints only size the LDS staging: with hints that are too small (tiles do not fit and
+    are decoded from global memory) or absent the result must not change."""
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant")
+    T, B, H, D, rep = 256, 1, 2, 128, 1
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    good = CompressedAttention(kctx, vctx).attend(q)
+    for c in (kctx, vctx):
+        if hint == "too_small":
+            c.max_tile_bytes, c.max_stream_bytes, c.max_code_bits = 16, 4, 1
+        else:
+            c.max_tile_bytes = c.max_stream_bytes = c.max_code_bits = 0
+    again = CompressedAttention(kctx, vctx).attend(q)
+    assert (again - good).abs().max() <= 1e-5 * good.abs().max()
