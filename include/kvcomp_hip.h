@@ -201,6 +201,13 @@ int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H,
               float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
               int64_t *d_counts, void *stream);
 
+/* ---- simulated quantization: quant_error (utils/compute.py:108-133), the value the reference's model caches
+ * keep (models/cache/kvcomp_quant.py:51-69): quant_ints followed by (quant_int + min_quant) * quant_scale,
+ * every step an fp16 tensor op on un-cast fp16 symbols and minima (so minima outside int8 do not wrap).
+ * d_xhat_f16 fp16, same shape and grouping rules as kvc_quant; nothing else is written. */
+int kvc_quant_error(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                    float eb, void *d_xhat_f16, void *stream);
+
 /* ---- dequantizer: (sym + min_i) * scale (models/cache/kvcomp_encode.py:146,161) --------------------
  * d_out fp16 = RN16(f32(sym + min_i) * f32(scale)), same shape as d_sym. */
 int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const void *d_scale_f16,

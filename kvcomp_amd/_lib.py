@@ -36,6 +36,7 @@ _SIGNATURES = {
     "kvc_k_mat_vec_mul": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_quant_groups": [_i64, _i64, _i64, _i64, _i64, _int],
     "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],
+    "kvc_quant_error": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp],
     "kvc_calibration_copy": [_vp, _vp, _i64, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }

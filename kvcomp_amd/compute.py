@@ -99,6 +99,49 @@ def dequant(quant_ints: torch.Tensor, min_ints: torch.Tensor, quant_scale: torch
     return out
 
 
+# Simulated quantization on the sim path's [B, H, NB, BS, D] view (utils/compute.py:74-91,108-133).  The groups
+# of ChannelQuant ([3]) and VectorQuant ([4]) are contiguous runs of that layout as it stands; BlockQuant
+# ([1, 3, 4]) and TokenQuant ([1, 4]) reduce over the head dimension, which has to sit inside the block first.
+_SIM_PLAN = {
+    QuantMode.ChannelQuant: (False, 0x1),
+    QuantMode.VectorQuant: (False, 0x8),
+    QuantMode.TokenQuant: (True, 0xC),
+    QuantMode.BlockQuant: (True, 0xD),
+}
+
+
+def quant_dequant_sim(tensor: torch.Tensor, block_size: int, quant_scale_rel: float, quant_mode: QuantMode) -> torch.Tensor:
+    """`(quant_int + min_quant) * quant_scale` of utils/compute.py:124-131 for a device fp16 [B, H, T, D] tensor
+    (T a multiple of block_size), bit-identical to the reference's chain of fp16 tensor ops, as one kernel."""
+    if tensor.dim() != 4 or tensor.dtype != torch.float16 or not tensor.is_cuda:
+        raise KvcompError("quant_dequant_sim expects a device float16 tensor of shape [B, H, T, D]")
+    B, H, T, D = tensor.shape
+    if T % block_size != 0:
+        raise KvcompError("Tensor shape is not divisible by block size")
+    heads_inside, mask = _SIM_PLAN[quant_mode]
+    NB = T // block_size
+    if heads_inside:
+        x = tensor.permute(0, 2, 1, 3).contiguous()                    # [B, T, H, D]
+        shape5 = (B * NB, block_size, 1, H, D)
+    else:
+        x = tensor.contiguous()
+        shape5 = (B * H * NB, block_size, 1, 1, D)
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        check(_lib.lib().kvc_quant_error(_ptr(x), *shape5, mask, float(quant_scale_rel), _ptr(out), _stream(x)))
+    return out.permute(0, 2, 1, 3) if heads_inside else out
+
+
+def quant_error(error_cache, buffer, new_tensor, block_size: int, recent_size: int, quant_scale_rel: float,
+                quant_mode: QuantMode):
+    """utils/compute.py:108-133: append to the tail, replace the whole blocks that leave it by their
+    simulated-quantization values and append those to `error_cache`."""
+    to_compress, in_buffer = cut_tensor(buffer, new_tensor, block_size, recent_size, dim=2)
+    if to_compress is not None:
+        to_compress = quant_dequant_sim(to_compress, block_size, quant_scale_rel, quant_mode)
+    return safe_cat(error_cache, to_compress, dim=2), in_buffer
+
+
 def safe_cat(t1, t2, dim):
     """utils/compute.py:35-42"""
     if t1 is None and t2 is None:

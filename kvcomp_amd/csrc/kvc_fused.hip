@@ -33,6 +33,8 @@
 // from LDS or -- for an oversized tile -- from global memory.
 #include "kvc_tile.h"
 
+#include <type_traits>
+
 struct KvcFusedArgs {
     KvcStreamArgs s;
     const int8_t *min_i8;
@@ -137,44 +139,61 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
 // is the entry's address.
 typedef __attribute__((address_space(3))) uint32_t kvc_lds_u32;
 
+// compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>)
+template <int N, int I = 0, class Body>
+__device__ __forceinline__ void kvc_static_for(Body &&body)
+{
+    if constexpr (I < N) {
+        body(std::integral_constant<int, I>{});
+        kvc_static_for<N, I + 1>(body);
+    }
+}
+
+// acc += x * (the value of `quad` in lane (l & ~3) + J of lane l's quad): the lane permute rides on the FMA's
+// first operand, so picking one of the four operands a quad holds costs no instruction of its own.
+// (`quad` comes straight from an LDS read and `acc` is not the permuted operand, so no VALU-write -> permuted-read
+// hazard can arise between consecutive FMAs.)
+template <int J>
+__device__ __forceinline__ void kvc_fma_quad_pick(float &acc, uint32_t quad, float x)
+{
+    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[%3,%3,%3,%3] row_mask:0xf bank_mask:0xf"
+        : "+v"(acc)
+        : "v"(quad), "v"(x), "n"(J));
+}
+
 template <int G, bool CHECK, int REP>
 __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t last_word, uint32_t &u,
                                              uint32_t fentry_base, uint32_t mask4, int n,
                                              const float *ops, float (&acc)[REP], uint32_t &worst)
 {
-#pragma unroll 2
+    const float *ops_q = ops + (__lane_id() & 3);
     for (int i = 0; i < n; i += G) {
         uint32_t a = u >> 5;
         a = a < last_word ? a : last_word;
         const uint32_t w0 = stage[a], w1 = stage[a + 1];
-        float op[G * REP];
-        if (G * REP >= 4) {
+        // The group's G * REP operands, four per register: lane l holds element l & 3 of each block of four
+        // and the FMA picks its operand from the right lane of the quad.  One 4-byte read per lane moves a
+        // quarter of what a 16-byte broadcast read of the same four values would.
+        constexpr int NBLK = (G * REP + 3) / 4;
+        uint32_t blk[NBLK];
 #pragma unroll
-            for (int k = 0; k < G * REP; k += 4) {
-                const float4 v = *reinterpret_cast<const float4 *>(ops + i * REP + k);
-                op[k] = v.x;
-                op[k + 1] = v.y;
-                op[k + 2] = v.z;
-                op[k + 3] = v.w;
-            }
-        } else {   // G = 2, REP = 1
-            const float2 v = *reinterpret_cast<const float2 *>(ops + i * REP);
-            op[0] = v.x;
-            op[1] = v.y;
-        }
+        for (int k = 0; k < NBLK; k++) blk[k] = __float_as_uint(ops_q[i * REP + 4 * k]);
         // 32 stream bits from bit u on: bits [1:0] are the pair before the lane's position, the next code
         // starts at bit 2
         uint32_t R = __builtin_amdgcn_alignbit(w1, w0, u);
         uint32_t es = 0;
-#pragma unroll
-        for (int g = 0; g < G; g++) {
+        kvc_static_for<G>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;
             const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
             R = __builtin_amdgcn_alignbit(R, R, e);                   // rotate right by len
             es += e;
             const float f = __uint_as_float(e);
-#pragma unroll
-            for (int r = 0; r < REP; r++) acc[r] = fmaf(f, op[g * REP + r], acc[r]);
-        }
+            kvc_static_for<REP>([&](auto r_) {
+                constexpr int r = decltype(r_)::value;
+                constexpr int k = g * REP + r;
+                kvc_fma_quad_pick<k & 3>(acc[r], blk[k >> 2], f);
+            });
+        });
         const uint32_t used = es & 0xffu;
         if (CHECK) worst = used > worst ? used : worst;
         u += used;
@@ -393,7 +412,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 }
 
 template <int REP, int KIND>
-__global__ void __launch_bounds__(KVC_WG, REP == 1 ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KIND != 2)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;

@@ -34,12 +34,25 @@ __device__ __forceinline__ KvcGroupParams kvc_group_params(float mn, float mx, f
     return g;
 }
 
-__device__ __forceinline__ uint8_t kvc_quant_one(float x, const KvcGroupParams &g)
+__device__ __forceinline__ __half kvc_quant_one_f16(float x, const KvcGroupParams &g)
 {
     const __half q = __float2half_rn(__fdiv_rn(x, g.scale));                // tensor / quant_scale
     const float qi = __half2float(__float2half_rn(rintf(__half2float(q)))); // .round_()
-    const __half s = __float2half_rn(qi - g.min_i);                         // quant_ints - min_ints
-    return (uint8_t)(int)__half2float(s);                                   // .to(torch.uint8)
+    return __float2half_rn(qi - g.min_i);                                   // quant_ints - min_ints
+}
+
+__device__ __forceinline__ uint8_t kvc_quant_one(float x, const KvcGroupParams &g)
+{
+    return (uint8_t)(int)__half2float(kvc_quant_one_f16(x, g));             // .to(torch.uint8)
+}
+
+// The value the simulated-quantization path keeps (utils/compute.py:130): (quant_int + min_quant) * quant_scale,
+// two fp16 tensor ops on the un-cast fp16 symbol and minimum.
+__device__ __forceinline__ __half kvc_quant_error_one(float x, const KvcGroupParams &g)
+{
+    const __half s = kvc_quant_one_f16(x, g);
+    const __half sum = __float2half_rn(__half2float(s) + g.min_i);
+    return __float2half_rn(__half2float(sum) * g.scale);
 }
 
 __device__ __forceinline__ float kvc_wave_min(float v)
@@ -75,8 +88,29 @@ struct KvcQuantArgs {
     int8_t *min_i8;
     __half *scale_f16;
     __half *min_f16;       // optional
+    __half *xhat;          // optional: simulated-quantization values, same shape as x
     uint32_t *minmax;      // block modes: {ord(min), ord(max)} per group
 };
+
+// Writes the symbols and/or the simulated-quantization values of two adjacent elements.
+__device__ __forceinline__ void kvc_quant_store2(const KvcQuantArgs &a, int64_t i, float v0, float v1,
+                                                 const KvcGroupParams &g0, const KvcGroupParams &g1)
+{
+    if (a.sym) {
+        uchar2 o;
+        o.x = kvc_quant_one(v0, g0);
+        o.y = kvc_quant_one(v1, g1);
+        *reinterpret_cast<uchar2 *>(a.sym + i) = o;
+    }
+    if (a.xhat) *reinterpret_cast<__half2 *>(a.xhat + i) = __halves2half2(kvc_quant_error_one(v0, g0), kvc_quant_error_one(v1, g1));
+}
+
+__device__ __forceinline__ void kvc_quant_publish(const KvcQuantArgs &a, int64_t g, const KvcGroupParams &gp)
+{
+    if (a.scale_f16) a.scale_f16[g] = gp.scale_h;
+    if (a.min_i8) a.min_i8[g] = (int8_t)(int)gp.min_i;
+    if (a.min_f16) a.min_f16[g] = gp.min_h;
+}
 
 // ---- per-channel groups (mask 0x1): a thread owns two adjacent channels of one block and walks the
 // BS tokens twice; no cross-lane traffic at all. ------------------------------------------------------
@@ -97,18 +131,12 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_kernel(KvcQuantArgs 
     }
     const KvcGroupParams g0 = kvc_group_params(mn0, mx0, a.eb), g1 = kvc_group_params(mn1, mx1, a.eb);
     const int64_t g = nb * stride + c;
-    a.scale_f16[g] = g0.scale_h;
-    a.scale_f16[g + 1] = g1.scale_h;
-    a.min_i8[g] = (int8_t)(int)g0.min_i;
-    a.min_i8[g + 1] = (int8_t)(int)g1.min_i;
-    if (a.min_f16) { a.min_f16[g] = g0.min_h; a.min_f16[g + 1] = g1.min_h; }
-    uint8_t *s = a.sym + nb * a.BS * stride + c;
+    kvc_quant_publish(a, g, g0);
+    kvc_quant_publish(a, g + 1, g1);
+    const int64_t base = nb * a.BS * stride + c;
     for (int64_t t = 0; t < a.BS; t++) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + t * stride);
-        uchar2 o;
-        o.x = kvc_quant_one(__low2float(v), g0);
-        o.y = kvc_quant_one(__high2float(v), g1);
-        *reinterpret_cast<uchar2 *>(s + t * stride) = o;
+        kvc_quant_store2(a, base + t * stride, __low2float(v), __high2float(v), g0, g1);
     }
 }
 
@@ -130,18 +158,10 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, i
     mn = kvc_wave_min(mn);
     mx = kvc_wave_max(mx);
     const KvcGroupParams gp = kvc_group_params(mn, mx, a.eb);
-    if (lane == 0) {
-        a.scale_f16[g] = gp.scale_h;
-        a.min_i8[g] = (int8_t)(int)gp.min_i;
-        if (a.min_f16) a.min_f16[g] = gp.min_h;
-    }
-    uint8_t *s = a.sym + g * R;
+    if (lane == 0) kvc_quant_publish(a, g, gp);
     for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
-        uchar2 o;
-        o.x = kvc_quant_one(__low2float(v), gp);
-        o.y = kvc_quant_one(__high2float(v), gp);
-        *reinterpret_cast<uchar2 *>(s + i) = o;
+        kvc_quant_store2(a, g * R + i, __low2float(v), __high2float(v), gp, gp);
     }
 }
 
@@ -191,19 +211,11 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_block_apply_kernel(KvcQuantA
     const KvcGroupParams gp = kvc_group_params(kvc_ord2f(a.minmax[2 * g]), kvc_ord2f(a.minmax[2 * g + 1]), a.eb);
     // the first row of a group also publishes the group's metadata
     const bool first = a.mask == KVC_MASK_K_BLOCK ? (row % a.BS == 0) : ((row / a.B) % a.BS == 0);
-    if (first && lane == 0) {
-        a.scale_f16[g] = gp.scale_h;
-        a.min_i8[g] = (int8_t)(int)gp.min_i;
-        if (a.min_f16) a.min_f16[g] = gp.min_h;
-    }
+    if (first && lane == 0) kvc_quant_publish(a, g, gp);
     const __half *p = a.x + row * R;
-    uint8_t *s = a.sym + row * R;
     for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
-        uchar2 o;
-        o.x = kvc_quant_one(__low2float(v), gp);
-        o.y = kvc_quant_one(__high2float(v), gp);
-        *reinterpret_cast<uchar2 *>(s + i) = o;
+        kvc_quant_store2(a, row * R + i, __low2float(v), __high2float(v), gp, gp);
     }
 }
 
@@ -214,14 +226,15 @@ extern "C" int64_t kvc_quant_groups(int64_t NB, int64_t BS, int64_t B, int64_t H
 
 extern "C" int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts, void *stream);
 
-extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
-                         float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
-                         int64_t *d_counts, void *stream_)
+static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                            float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
+                            void *d_xhat_f16, int64_t *d_counts, void *stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     KVC_REQUIRE(NB >= 0 && BS > 0 && B > 0 && H > 0 && D > 0, "bad shape");
     KVC_REQUIRE(D % 2 == 0, "head_dim must be even");
-    KVC_REQUIRE(((uintptr_t)d_x_f16 & 3) == 0 && ((uintptr_t)d_sym & 1) == 0, "quantizer buffers are misaligned");
+    KVC_REQUIRE(((uintptr_t)d_x_f16 & 3) == 0 && ((uintptr_t)d_sym & 1) == 0 && ((uintptr_t)d_xhat_f16 & 3) == 0,
+                "quantizer buffers are misaligned");
     KVC_REQUIRE(eb > 0.f, "error bound must be positive");
     if (NB == 0) return 0;
     KvcQuantArgs a;
@@ -233,6 +246,7 @@ extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B,
     a.min_i8 = d_min_i8;
     a.scale_f16 = reinterpret_cast<__half *>(d_scale_f16);
     a.min_f16 = reinterpret_cast<__half *>(d_min_f16);
+    a.xhat = reinterpret_cast<__half *>(d_xhat_f16);
     a.minmax = nullptr;
     const int64_t stride = B * H * D;
     if (quant_mask == KVC_MASK_CHANNEL) {
@@ -261,6 +275,23 @@ extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B,
     KVC_HIP(hipGetLastError());
     if (d_counts) return kvc_histogram(d_sym, NB * BS * stride, d_counts, stream_);
     return 0;
+}
+
+extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                         float eb, uint8_t *d_sym, int8_t *d_min_i8, void *d_scale_f16, void *d_min_f16,
+                         int64_t *d_counts, void *stream)
+{
+    KVC_REQUIRE(d_sym != nullptr && d_min_i8 != nullptr && d_scale_f16 != nullptr, "output pointer is NULL");
+    return kvc_quant_launch(d_x_f16, NB, BS, B, H, D, quant_mask, eb, d_sym, d_min_i8, d_scale_f16, d_min_f16, nullptr,
+                            d_counts, stream);
+}
+
+extern "C" int kvc_quant_error(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                               float eb, void *d_xhat_f16, void *stream)
+{
+    KVC_REQUIRE(d_xhat_f16 != nullptr, "output pointer is NULL");
+    return kvc_quant_launch(d_x_f16, NB, BS, B, H, D, quant_mask, eb, nullptr, nullptr, nullptr, nullptr, d_xhat_f16,
+                            nullptr, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------

@@ -255,7 +255,10 @@ class KVCompCtx:
         return out.flatten(0, 1), t_ms + start.elapsed_time(end)
 
     def get(self) -> Tuple[torch.Tensor, float]:
-        """kvcomp_encode.py:138-151: compressed part followed by the uncompressed tail."""
+        """kvcomp_encode.py:138-151: compressed part followed by the uncompressed tail.  (While nothing has
+        been compressed yet the tail is everything; the reference asserts in that state.)"""
+        if self.compressed_ctx_len == 0:
+            return self.buffer, 0.0
         out, t_ms = self.get_only_compressed()
         if self.buffer is not None and self.buffer.shape[0] > 0:
             out = torch.cat([out, self.buffer], dim=0)
