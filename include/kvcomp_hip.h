@@ -182,6 +182,44 @@ int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook, const uint
                        int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                        float *elapsed_ms, void *stream);
 
+/* ---- decode attention in one call (no counterpart in the reference: its models decompress the whole cache and
+ * run dense attention, models/cache/kvcomp_quant.py:74-75) ----------------------------------------------------
+ * out[b, hq, :] = softmax_t(softmax_scale * q[b, hq, :] . K[t, b, h, :]) . V[t, b, h, :] over every stored token:
+ * the compressed parts of K and V through the fused kernels, their fp16 tails (the most recent tokens, which K
+ * and V keep in different numbers) densely.  A kvc_compressed_desc describes one tensor of the pair: the same
+ * arrays the other entry points take (layout of models/cache/kvcomp_encode.py:15-67), the decode tables from
+ * kvc_build_lut, the encoder's size hints (0 = unknown), `tokens` compressed tokens (a multiple of 64 for K,
+ * 128 for V) and `tail_tokens` fp16 tokens [tail, batch, kv_heads, head_dim] that follow them.
+ * d_workspace: kvc_attention_workspace_bytes(...) bytes of device memory, 256-byte aligned, contents ignored.
+ * d_out_f32: fp32 [batch, q_heads, head_dim].
+ * fused_kernel_ms (may be NULL): receives the durations of the fused K and fused V kernels; asking for them
+ * makes the call wait for each of the two kernels. */
+typedef struct kvc_compressed_desc {
+    const void *d_luts;
+    int64_t rows_per_codebook;
+    const uint8_t *d_block_infos;
+    int64_t block_infos_bytes;
+    const uint8_t *d_thread_infos;
+    int64_t thread_infos_bytes;
+    const uint8_t *d_encoded;
+    int64_t encoded_bytes;
+    const int8_t *d_quant_min_ints;
+    const void *d_quant_scales_f16;
+    int64_t quant_mask;
+    int64_t max_tile_bytes;
+    int64_t max_stream_bytes;
+    int64_t max_code_bits;
+    int64_t tokens;
+    const void *d_tail_f16;
+    int64_t tail_tokens;
+} kvc_compressed_desc;
+int64_t kvc_attention_workspace_bytes(int64_t total_tokens, int64_t v_compressed_tokens, int64_t batch,
+                                      int64_t q_heads, int64_t head_dim);
+int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                         float softmax_scale, void *d_workspace, int64_t workspace_bytes, float *d_out_f32,
+                         int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                         float *elapsed_ms, float *fused_kernel_ms, void *stream);
+
 /* ---- dense baseline: k_mat_vec_mul_cuda_export (kernels.cu:1182-1273) ------------------------------
  * d_k fp16 [tokens, batch, heads, head_dim], d_q fp16 [batch, heads, head_dim],
  * d_out fp16 [tokens, batch, heads].  (The reference requires batch == 1 and head_dim == 128.) */

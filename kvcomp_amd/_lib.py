@@ -12,6 +12,18 @@ _LIB = None
 _i64, _int, _vp, _f32p, _u32 = C.c_int64, C.c_int, C.c_void_p, C.POINTER(C.c_float), C.c_uint32
 _i64p, _intp = C.POINTER(C.c_int64), C.POINTER(C.c_int)
 
+class CompressedDesc(C.Structure):
+    """kvc_compressed_desc of include/kvcomp_hip.h."""
+    _fields_ = [("d_luts", C.c_void_p), ("rows_per_codebook", C.c_int64),
+                ("d_block_infos", C.c_void_p), ("block_infos_bytes", C.c_int64),
+                ("d_thread_infos", C.c_void_p), ("thread_infos_bytes", C.c_int64),
+                ("d_encoded", C.c_void_p), ("encoded_bytes", C.c_int64),
+                ("d_quant_min_ints", C.c_void_p), ("d_quant_scales_f16", C.c_void_p),
+                ("quant_mask", C.c_int64), ("max_tile_bytes", C.c_int64), ("max_stream_bytes", C.c_int64),
+                ("max_code_bits", C.c_int64), ("tokens", C.c_int64),
+                ("d_tail_f16", C.c_void_p), ("tail_tokens", C.c_int64)]
+
+
 # name -> argtypes (every function returns int unless listed in _RESTYPES)
 _SIGNATURES = {
     "kvc_abi_version": [],
@@ -38,9 +50,12 @@ _SIGNATURES = {
     "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],
     "kvc_quant_error": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp],
     "kvc_calibration_copy": [_vp, _vp, _i64, _vp],
+    "kvc_attention_workspace_bytes": [_i64, _i64, _i64, _i64, _i64],
+    "kvc_attention_decode": [C.POINTER(CompressedDesc), C.POINTER(CompressedDesc), _vp, C.c_float, _vp, _i64, _vp,
+                             _i64, _i64, _i64, _i64, _f32p, _f32p, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }
-_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64}
+_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_attention_workspace_bytes": _i64}
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["kvc_last_error"])
 

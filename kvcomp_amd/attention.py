@@ -81,12 +81,15 @@ class CompressedAttention:
         self.k, self.v = k_ctx, v_ctx
         self._k_lut = self._v_lut = None
         self._k_lut_src = self._v_lut_src = None
+        self._workspace = None
+        self._keep = []
 
     def _luts(self):
         # decode tables follow the contexts' codebooks (built once, rebuilt if a codebook is replaced)
-        if self._k_lut is None or self._k_lut_src is not self.k.decode_codebook:
+        # (a context has no codebook until its first block is compressed)
+        if self.k.decode_codebook is not None and self._k_lut_src is not self.k.decode_codebook:
             self._k_lut, self._k_lut_src = build_lut(self.k.decode_codebook), self.k.decode_codebook
-        if self._v_lut is None or self._v_lut_src is not self.v.decode_codebook:
+        if self.v.decode_codebook is not None and self._v_lut_src is not self.v.decode_codebook:
             self._v_lut, self._v_lut_src = build_lut(self.v.decode_codebook), self.v.decode_codebook
         return self._k_lut, self._v_lut
 
@@ -104,8 +107,55 @@ class CompressedAttention:
         if ev is not None:
             ev.record()
 
-    def attend(self, q: torch.Tensor, scale: Optional[float] = None, prof: Optional[dict] = None) -> torch.Tensor:
-        """q fp16 [B, Hq, D] -> fp32 [B, Hq, D].  Covers every stored token: the compressed part through the
+    def _desc(self, ctx: KVCompCtx, lut) -> "_lib.CompressedDesc":
+        d = _lib.CompressedDesc()
+        if ctx.compressed_ctx_len:
+            d.d_luts = lut.data_ptr()
+            d.d_block_infos, d.block_infos_bytes = ctx.block_infos.data_ptr(), ctx.block_infos.numel()
+            d.d_thread_infos, d.thread_infos_bytes = ctx.thread_infos.data_ptr(), ctx.thread_infos.numel()
+            d.d_encoded, d.encoded_bytes = ctx.encoded_data.data_ptr(), ctx.encoded_data.numel()
+            d.d_quant_min_ints, d.d_quant_scales_f16 = ctx.quant_min_ints.data_ptr(), ctx.quant_scales.data_ptr()
+        d.rows_per_codebook = 0
+        d.quant_mask = dims_to_mask(ctx.quant_dims)
+        d.max_tile_bytes, d.max_stream_bytes, d.max_code_bits = ctx.max_tile_bytes, ctx.max_stream_bytes, ctx.max_code_bits
+        d.tokens = ctx.compressed_ctx_len
+        tail = ctx.buffer
+        d.tail_tokens = 0 if tail is None else tail.shape[0]
+        if d.tail_tokens:
+            self._keep.append(tail.contiguous())
+            d.d_tail_f16 = self._keep[-1].data_ptr()
+        return d
+
+    def attend(self, q: torch.Tensor, scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+               kernel_ms: Optional[list] = None) -> torch.Tensor:
+        """q fp16 [B, Hq, D] -> fp32 [B, Hq, D] over every stored token, as one library call
+        (kvc_attention_decode): scores, softmax and the weighted sum of values never pass through PyTorch.
+        `kernel_ms`, if a list, receives (fused K kernel ms, fused V kernel ms) -- which makes the call wait."""
+        B, Hq, D = q.shape
+        assert q.dtype == torch.float16 and self.v.ctx_len == self.k.ctx_len
+        scale = scale if scale is not None else 1.0 / math.sqrt(D)
+        k_lut, v_lut = self._luts()
+        L = _lib.lib()
+        need = int(L.kvc_attention_workspace_bytes(self.k.ctx_len, self.v.compressed_ctx_len, B, Hq, D))
+        if self._workspace is None or self._workspace.numel() < need or self._workspace.device != q.device:
+            self._workspace = torch.empty(need + need // 4, dtype=torch.uint8, device=q.device)
+        if out is None:
+            out = torch.empty(B, Hq, D, dtype=torch.float32, device=q.device)
+        self._keep = []
+        kd, vd = self._desc(self.k, k_lut), self._desc(self.v, v_lut)
+        q = q.contiguous()
+        ms = (C.c_float * 2)()
+        with torch.cuda.device(q.device):
+            check(L.kvc_attention_decode(C.byref(kd), C.byref(vd), _ptr(q), float(scale), _ptr(self._workspace),
+                                         self._workspace.numel(), _ptr(out), B, self.k.head_num, Hq, D, None,
+                                         ms if kernel_ms is not None else None, _stream(q.device)))
+        if kernel_ms is not None:
+            kernel_ms[:] = [float(ms[0]), float(ms[1])]
+        return out
+
+    def attend_stepwise(self, q: torch.Tensor, scale: Optional[float] = None, prof: Optional[dict] = None) -> torch.Tensor:
+        """The same result assembled from the reference-shaped pieces (fused K scores, PyTorch softmax, fused
+        p.V partials, PyTorch reduction).  q fp16 [B, Hq, D] -> fp32 [B, Hq, D].  Covers every stored token: the compressed part through the
         fused kernels, the fp16 tails (K and V compress on different block sizes, so their tails differ)
         through dense matvecs.  `prof`, if given, collects (start, end) event pairs recorded on the launch
         stream around the two fused kernels under the keys "k" and "v"."""

@@ -151,6 +151,13 @@ __device__ __forceinline__ float kvc_wave_sum_dpp(float v)
     }));
 }
 
+__device__ __forceinline__ float kvc_wave_fmax_dpp(float v)
+{
+    return __uint_as_float(kvc_wave_reduce_dpp(__float_as_uint(v), [](uint32_t a, uint32_t b) {
+        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
+    }));
+}
+
 __device__ __forceinline__ uint32_t kvc_wave_max_dpp(uint32_t v)
 {
     return kvc_wave_reduce_dpp(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; });

@@ -43,6 +43,14 @@ struct KvcFusedArgs {
     const __half *x;     // K: q [batch, q_heads, head_dim];  V: p [batch, q_heads, tokens]
     void *out;           // K: scores [batch, q_heads, tokens]; V: partial [tokens/128, batch, q_heads, head_dim]
     int out_f32;         // 0: fp16 (reference layout), 1: fp32
+    int64_t out_stride;  // K: elements between the score rows of two query heads (>= tokens)
+    // softmax kinds of the V kernel: instead of p it reads raw fp32 scores and forms, per 128-token group and
+    // query head, m = max(score * sm_scale), w = exp(score * sm_scale - m), l = sum w; the partial is the
+    // w-weighted sum and (m, l) go to ml[group][batch][q_head][2]
+    const float *scores;
+    int64_t scores_stride;
+    float sm_scale;
+    float *ml;
     int64_t tokens;
     int batch, kv_heads, q_heads, head_dim;
     int table_words;     // LDS words reserved for the fused table (>= 1 << lbits of every codebook used)
@@ -54,7 +62,7 @@ constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one til
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
 
 // What a tile needs from global memory, fetched into registers one tile ahead of its use.
-template <int REP, int SLOTS>
+template <int REP, int SLOTS, int XW>
 struct KvcRaw {
     uint4 pay[KVC_PRE_CHUNKS];        // payload chunks lane, lane + 64, ...
     uint32_t off, bn;                 // block_info, clamped to the payload buffer (wave-uniform)
@@ -62,7 +70,7 @@ struct KvcRaw {
     // operands of elements 2 * lane and 2 * lane + 1 (K: channels, V: tokens of the 128-token group), as loaded:
     uint16_t sc[SLOTS][2];            // quantization scale (fp16 bits)
     int8_t mn[SLOTS][2];              // quantization minimum
-    uint32_t x[SLOTS][REP];           // q / p (two fp16), per query head
+    uint32_t x[SLOTS][REP][XW];       // per query head: q / p (two fp16 in one word), or two fp32 scores
 };
 // Nothing in it is touched before the tile is staged: any arithmetic on a loaded value would make the wave
 // wait for the load at that point and the fetch would no longer overlap the decode of the previous tile.
@@ -204,16 +212,19 @@ __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t las
 // KIND 0: K tile (64 tokens x head_dim channels of one (batch, head); lane = token)
 // KIND 1: V tile (128 tokens x 64 flat channels; lane = channel), head_dim a multiple of 64: one head per tile
 // KIND 2: V tile with any other head_dim: the 64 channels may straddle two heads (two operand tables)
+// KIND 3, 4: as 1, 2 but with the softmax over the group's scores computed on the fly
 template <int KIND>
 struct KvcGeom {
     static constexpr bool IS_K = KIND == 0;
-    static constexpr int SLOTS = KIND == 2 ? 2 : 1;
+    static constexpr int SLOTS = (KIND == 2 || KIND == 4) ? 2 : 1;
+    static constexpr bool SOFTMAX = KIND >= 3;
+    static constexpr int XW = SOFTMAX ? 2 : 1;
 };
 
 // Issue the global loads of tile (row, col).  bi_off / bi_bn: the tile's block_info words.
 template <int REP, int KIND>
 __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
-                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS> &raw)
+                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     const int64_t tile = (int64_t)row * a.s.cols + col;
@@ -253,7 +264,7 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
         }
 #pragma unroll
         for (int r = 0; r < REP; r++)
-            raw.x[0][r] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
+            raw.x[0][r][0] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
     } else {
         const int bh0 = (col * KVC_WAVE) / D;
         const int bh_max = a.batch * a.kv_heads - 1;
@@ -273,8 +284,16 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
                 raw.mn[s][half] = a.min_i8[g];
             }
 #pragma unroll
-            for (int r = 0; r < REP; r++)
-                raw.x[s][r] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * a.tokens + tk);
+            for (int r = 0; r < REP; r++) {
+                const int64_t xrow = (int64_t)b * a.q_heads + h * REP + r;
+                if (KvcGeom<KIND>::SOFTMAX) {
+                    const uint2 v = *reinterpret_cast<const uint2 *>(a.scores + xrow * a.scores_stride + tk);
+                    raw.x[s][r][0] = v.x;
+                    raw.x[s][r][KvcGeom<KIND>::XW - 1] = v.y;
+                } else {
+                    raw.x[s][r][0] = *reinterpret_cast<const uint32_t *>(a.x + xrow * a.tokens + tk);
+                }
+            }
         }
     }
 }
@@ -296,7 +315,7 @@ struct KvcStaged {
 // constant terms sum_i min_i * operand_i in bias[].
 template <int REP, int KIND>
 __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int row, int col, int lane,
-                                                    const KvcRaw<REP, KvcGeom<KIND>::SLOTS> &raw, float *ops,
+                                                    const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw, float *ops,
                                                     uint32_t *pack, uint32_t *rows, float (&bias)[REP], int &sel_out)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
@@ -360,6 +379,30 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 #pragma unroll
         for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f;
         const bool live = KIND != 0 || 2 * lane < D;
+        float wgt[REP][2];                           // the two elements' weights: q, p, or exp(score - max)
+#pragma unroll
+        for (int r = 0; r < REP; r++) {
+            if (KvcGeom<KIND>::SOFTMAX) {
+                const float s0 = __uint_as_float(raw.x[s][r][0]) * a.sm_scale;
+                const float s1 = __uint_as_float(raw.x[s][r][KvcGeom<KIND>::XW - 1]) * a.sm_scale;
+                const float m = kvc_wave_fmax_dpp(fmaxf(s0, s1));
+                wgt[r][0] = __expf(s0 - m);
+                wgt[r][1] = __expf(s1 - m);
+                const float l = kvc_wave_sum_dpp(wgt[r][0] + wgt[r][1]);
+                if (lane == 0) {
+                    int bh = (col * KVC_WAVE) / D + s;
+                    const int bh_max = a.batch * a.kv_heads - 1;
+                    bh = bh < bh_max ? bh : bh_max;
+                    const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
+                    float *ml = a.ml + (((int64_t)row * a.batch + b) * a.q_heads + h * REP + r) * 2;
+                    ml[0] = m;     // tiles that share a head write the same pair
+                    ml[1] = l;
+                }
+            } else {
+                wgt[r][0] = kvc_half_bits_to_float(raw.x[s][r][0] & 0xffffu);
+                wgt[r][1] = kvc_half_bits_to_float(raw.x[s][r][0] >> 16);
+            }
+        }
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const int i = 2 * lane + half;
@@ -367,7 +410,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
             const float mn = (float)raw.mn[s][half];
 #pragma unroll
             for (int r = 0; r < REP; r++) {
-                const float v = sc * kvc_half_bits_to_float((raw.x[s][r] >> (16 * half)) & 0xffffu);
+                const float v = sc * wgt[r][half];
                 ops[(s * 128 + i) * REP + r] = v;
                 bias_s[s][r] += mn * v;
             }
@@ -376,7 +419,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
         for (int r = 0; r < REP; r++) bias_s[s][r] = kvc_wave_sum_dpp(bias_s[s][r]);
     }
     int sel = 0;
-    if (KIND == 2) {
+    if (SLOTS == 2) {
         const int c0 = col * KVC_WAVE;
         sel = (c0 % D + lane) >= D;                                        // 1 past a head boundary
     }
@@ -412,7 +455,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 }
 
 template <int REP, int KIND>
-__global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KIND != 2)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND>::SLOTS == 1)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
@@ -455,7 +498,7 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KIND != 2)) 
         bi_off = bi[0];
         bi_bn = bi[1];
     }
-    KvcRaw<REP, SLOTS> raw;
+    KvcRaw<REP, SLOTS, KvcGeom<KIND>::XW> raw;
     kvc_fetch_tile<REP, KIND>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
     float bias[REP];
     int sel = 0;
@@ -504,12 +547,12 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KIND != 2)) 
         int64_t out_base, out_step;
         if (IS_K) {
             const int b = col / a.kv_heads, h = col - b * a.kv_heads;
-            out_base = ((int64_t)b * a.q_heads + h * REP) * a.tokens + (int64_t)row * KVC_WAVE + lane;
-            out_step = a.tokens;
+            out_base = ((int64_t)b * a.q_heads + h * REP) * a.out_stride + (int64_t)row * KVC_WAVE + lane;
+            out_step = a.out_stride;
         } else {
             const int c0 = col * KVC_WAVE;
             const int bh0 = c0 / D, d0 = c0 - bh0 * D;                  // wave-uniform
-            const int past = (KIND == 2 && d0 + lane >= D) ? 1 : 0;     // this lane's channel lies in the next head
+            const int past = (SLOTS == 2 && d0 + lane >= D) ? 1 : 0;     // this lane's channel lies in the next head
             const int bh = bh0 + past, d = d0 + lane - past * D;
             const int b0 = bh0 / a.kv_heads, h0 = bh0 - b0 * a.kv_heads;
             const int wrap = (h0 + past == a.kv_heads) ? 1 : 0;         // ... which may be the first head of the next batch entry
@@ -540,7 +583,9 @@ static void kvc_launch_fused(int kind, const KvcFusedArgs &a, dim3 grid, size_t 
 {
     if (kind == 0) hipLaunchKernelGGL((kvc_fused_kernel<REP, 0>), grid, dim3(KVC_WG), lds, stream, a);
     else if (kind == 1) hipLaunchKernelGGL((kvc_fused_kernel<REP, 1>), grid, dim3(KVC_WG), lds, stream, a);
-    else hipLaunchKernelGGL((kvc_fused_kernel<REP, 2>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 2) hipLaunchKernelGGL((kvc_fused_kernel<REP, 2>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 3) hipLaunchKernelGGL((kvc_fused_kernel<REP, 3>), grid, dim3(KVC_WG), lds, stream, a);
+    else hipLaunchKernelGGL((kvc_fused_kernel<REP, 4>), grid, dim3(KVC_WG), lds, stream, a);
 }
 
 // LDS layout of one workgroup: the fused table, then per wave the operand table(s), the packed payload of
@@ -598,13 +643,23 @@ static int kvc_plan_tiles_per_wave(int64_t tiles)
     return tiles >= 2 * 256 * 4 * 5 ? 2 : 1;
 }
 
+// what the one-call attention adds to a plain fused launch
+struct KvcFusedExtra {
+    int64_t out_stride;          // K: row stride of the score matrix (0 = tokens)
+    const float *scores;         // V: fp32 scores in place of p (softmax on the fly), or NULL
+    int64_t scores_stride;
+    float sm_scale;
+    float *ml;
+};
+
 static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
                      const uint8_t *d_block_infos, int64_t block_infos_bytes, const uint8_t *d_thread_infos,
                      int64_t thread_infos_bytes, const uint8_t *d_encoded, int64_t encoded_bytes,
                      const int8_t *d_min, const void *d_scale, int quant_mask, const void *d_x, void *d_out,
                      int64_t tokens, int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                      float *elapsed_ms, void *stream_, const uint32_t *d_luts = nullptr, int rows_per_codebook = 0,
-                     int out_f32 = 0, int64_t max_tile_bytes = 0, int64_t max_stream_bytes = 0, int max_code_bits = 0)
+                     int out_f32 = 0, int64_t max_tile_bytes = 0, int64_t max_stream_bytes = 0, int max_code_bits = 0,
+                     const KvcFusedExtra *extra = nullptr)
 {
     hipStream_t stream = (hipStream_t)stream_;
     if (tokens == 0) {
@@ -639,13 +694,19 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     a.x = reinterpret_cast<const __half *>(d_x);
     a.out = d_out;
     a.out_f32 = out_f32;
+    a.out_stride = (extra && extra->out_stride) ? extra->out_stride : tokens;
+    a.scores = extra ? extra->scores : nullptr;
+    a.scores_stride = extra ? extra->scores_stride : 0;
+    a.sm_scale = extra ? extra->sm_scale : 1.f;
+    a.ml = extra ? extra->ml : nullptr;
     a.tokens = tokens;
     a.batch = (int)batch;
     a.kv_heads = (int)kv_heads;
     a.q_heads = (int)q_heads;
     a.head_dim = (int)head_dim;
-    const int kind = is_k ? 0 : (head_dim % KVC_WAVE == 0 ? 1 : 2);
-    const size_t lds = kvc_plan_lds(a, kind == 2 ? 2 : 1, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
+    const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
+    const int kind = is_k ? 0 : (a.scores ? 2 : 0) + slots;
+    const size_t lds = kvc_plan_lds(a, slots, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
                                     max_stream_bytes, max_code_bits);
     a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
     KvcTimer timer(elapsed_ms, stream);
@@ -731,4 +792,227 @@ extern "C" int kvc_v_partials_lut(const void *d_luts, int64_t rows_per_codebook,
                      d_encoded, encoded_bytes, d_quant_min_ints, d_quant_scales_f16, quant_mask, d_p_f16, d_partial, tokens,
                      batch, kv_heads, q_heads, head_dim, elapsed_ms, stream, (const uint32_t *)d_luts,
                      (int)rows_per_codebook, out_f32, max_tile_bytes, max_stream_bytes, max_code_bits);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// one-call decode attention over a compressed cache (no counterpart in the reference, whose models
+// decompress everything and run dense attention; models/cache/kvcomp_quant.py:74-75)
+//
+//   scores  = q . K^T        compressed part: fused K kernel; fp16 tail: kvc_tail_scores_kernel
+//   groups  of 128 tokens    compressed part: fused V kernel in softmax mode -> (m_g, l_g, sum_t w_t v_t);
+//                            fp16 tail: kvc_tail_values_kernel -> one more group
+//   out     = sum_g e^(m_g - M) part_g / sum_g e^(m_g - M) l_g          kvc_attention_combine_kernel
+//
+// Every 128-token group carries its own running maximum, so no pass over all scores is needed before the
+// values are read (the split-softmax scheme of flash decoding).
+// ---------------------------------------------------------------------------------------------------
+
+// scores[b, hq, t0 + t] = sum_d tail[t, b, h, d] q[b, hq, d]; one wave per (t, b, h), lanes over d
+__global__ void __launch_bounds__(KVC_WG)
+kvc_tail_scores_kernel(const __half *__restrict__ tail, const __half *__restrict__ q, float *__restrict__ scores,
+                       int64_t scores_stride, int64_t t0, int64_t tail_tokens, int batch, int kv_heads, int rep, int D)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t item = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
+    if (item >= tail_tokens * batch * kv_heads) return;
+    const int h = (int)(item % kv_heads);
+    const int b = (int)((item / kv_heads) % batch);
+    const int64_t t = item / ((int64_t)kv_heads * batch);
+    const __half *kp = tail + item * D;
+    float k0 = 0.f, k1 = 0.f;
+    if (2 * lane < D) {
+        const __half2 v = *reinterpret_cast<const __half2 *>(kp + 2 * lane);
+        k0 = __low2float(v);
+        k1 = __high2float(v);
+    }
+    for (int r = 0; r < rep; r++) {
+        const int hq = h * rep + r;
+        const __half *qp = q + ((int64_t)b * kv_heads * rep + hq) * D;
+        float acc = 0.f;
+        if (2 * lane < D) {
+            const __half2 v = *reinterpret_cast<const __half2 *>(qp + 2 * lane);
+            acc = k0 * __low2float(v) + k1 * __high2float(v);
+        }
+        acc = kvc_wave_sum_dpp(acc);
+        if (lane == 0) scores[((int64_t)b * kv_heads * rep + hq) * scores_stride + t0 + t] = acc;
+    }
+}
+
+// The tail tokens [t0, t0 + n) as one more group: one workgroup per (b, hq); thread d accumulates channel d.
+__global__ void __launch_bounds__(128)
+kvc_tail_values_kernel(const __half *__restrict__ tail, const float *__restrict__ scores, int64_t scores_stride,
+                       float sm_scale, float *__restrict__ part, float *__restrict__ ml, int64_t t0, int64_t n,
+                       int batch, int kv_heads, int rep, int D)
+{
+    const int hq = blockIdx.x % (kv_heads * rep), b = blockIdx.x / (kv_heads * rep);
+    const int h = hq / rep;
+    const float *sp = scores + ((int64_t)b * kv_heads * rep + hq) * scores_stride + t0;
+    float m = -INFINITY;
+    for (int64_t t = 0; t < n; t++) m = fmaxf(m, sp[t] * sm_scale);
+    float l = 0.f, acc = 0.f;
+    const int d = threadIdx.x;
+    for (int64_t t = 0; t < n; t++) {
+        const float w = __expf(sp[t] * sm_scale - m);
+        l += w;
+        if (d < D) acc += w * __half2float(tail[((t * batch + b) * kv_heads + h) * D + d]);
+    }
+    if (d < D) part[((int64_t)b * kv_heads * rep + hq) * D + d] = acc;
+    if (d == 0) {
+        ml[((int64_t)b * kv_heads * rep + hq) * 2] = m;
+        ml[((int64_t)b * kv_heads * rep + hq) * 2 + 1] = l;
+    }
+}
+
+// out[b, hq, :] from `groups` partials; one workgroup of 16 waves per (b, hq), wave w takes groups w, w + 16, ...
+constexpr int KVC_COMBINE_WAVES = 16;
+__global__ void __launch_bounds__(KVC_COMBINE_WAVES * KVC_WAVE)
+kvc_attention_combine_kernel(const float *__restrict__ part, const float *__restrict__ ml, int64_t groups,
+                             int64_t bhq_count, int D, float *__restrict__ out)
+{
+    __shared__ float s_max[KVC_COMBINE_WAVES];
+    __shared__ float s_num[KVC_COMBINE_WAVES][128];
+    __shared__ float s_den[KVC_COMBINE_WAVES];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t bhq = blockIdx.x;
+    // global maximum
+    float m = -INFINITY;
+    for (int64_t g = threadIdx.x; g < groups; g += KVC_COMBINE_WAVES * KVC_WAVE) m = fmaxf(m, ml[(g * bhq_count + bhq) * 2]);
+    m = kvc_wave_fmax_dpp(m);
+    if (lane == 0) s_max[wave] = m;
+    __syncthreads();
+    float M = s_max[0];
+#pragma unroll
+    for (int w = 1; w < KVC_COMBINE_WAVES; w++) M = fmaxf(M, s_max[w]);
+    float n0 = 0.f, n1 = 0.f, den = 0.f;
+    constexpr int U = 4;                                  // groups in flight per wave
+    for (int64_t g0 = wave; g0 < groups; g0 += U * KVC_COMBINE_WAVES) {
+        float mg[U], lg[U], p0[U], p1[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int64_t g = g0 + u * KVC_COMBINE_WAVES;
+            mg[u] = -INFINITY;
+            lg[u] = p0[u] = p1[u] = 0.f;
+            if (g < groups) {
+                const float *mlp = ml + (g * bhq_count + bhq) * 2;
+                const float *pp = part + (g * bhq_count + bhq) * D;
+                mg[u] = mlp[0];
+                lg[u] = mlp[1];
+                if (lane < D) p0[u] = pp[lane];
+                if (lane + 64 < D) p1[u] = pp[lane + 64];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const float f = __expf(mg[u] - M);             // exp(-inf) = 0 for the slots past the end
+            den += f * lg[u];
+            n0 += f * p0[u];
+            n1 += f * p1[u];
+        }
+    }
+    s_num[wave][lane] = n0;
+    s_num[wave][lane + 64] = n1;
+    if (lane == 0) s_den[wave] = den;
+    __syncthreads();
+    if (threadIdx.x < D) {
+        const int d = threadIdx.x;
+        float num = 0.f, dn = 0.f;
+#pragma unroll
+        for (int w = 0; w < KVC_COMBINE_WAVES; w++) {
+            num += s_num[w][d];
+            dn += s_den[w];
+        }
+        out[bhq * D + d] = num / dn;
+    }
+}
+
+static int64_t kvc_round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+struct KvcAttentionPlan {
+    int64_t total_tokens, scores_stride, groups;
+    int64_t scores_off, part_off, ml_off, bytes;
+};
+
+static KvcAttentionPlan kvc_attention_plan(int64_t total_tokens, int64_t v_compressed_tokens, int64_t batch, int64_t q_heads,
+                                           int64_t head_dim)
+{
+    KvcAttentionPlan p;
+    p.total_tokens = total_tokens;
+    p.scores_stride = kvc_round_up(total_tokens, 4);
+    p.groups = v_compressed_tokens / KVC_V_TOKENS + (total_tokens > v_compressed_tokens ? 1 : 0);
+    p.scores_off = 0;
+    p.part_off = kvc_round_up(batch * q_heads * p.scores_stride * 4, 256);
+    p.ml_off = p.part_off + kvc_round_up(p.groups * batch * q_heads * head_dim * 4, 256);
+    p.bytes = p.ml_off + kvc_round_up(p.groups * batch * q_heads * 2 * 4, 256);
+    return p;
+}
+
+extern "C" int64_t kvc_attention_workspace_bytes(int64_t total_tokens, int64_t v_compressed_tokens, int64_t batch,
+                                                 int64_t q_heads, int64_t head_dim)
+{
+    if (total_tokens <= 0 || v_compressed_tokens < 0 || batch <= 0 || q_heads <= 0 || head_dim <= 0) return 0;
+    return kvc_attention_plan(total_tokens, v_compressed_tokens, batch, q_heads, head_dim).bytes;
+}
+
+extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                                    float softmax_scale, void *d_workspace, int64_t workspace_bytes, float *d_out_f32,
+                                    int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                                    float *elapsed_ms, float *fused_kernel_ms, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    if (fused_kernel_ms) fused_kernel_ms[0] = fused_kernel_ms[1] = 0.f;
+    KVC_REQUIRE(k != nullptr && v != nullptr && d_q_f16 != nullptr && d_out_f32 != nullptr, "NULL argument");
+    KVC_REQUIRE(batch > 0 && kv_heads > 0 && q_heads > 0 && q_heads % kv_heads == 0, "q_heads must be a multiple of kv_heads");
+    KVC_REQUIRE(head_dim > 0 && head_dim <= 128 && head_dim % 8 == 0, "head_dim must be a multiple of 8, <= 128");
+    const int64_t total = k->tokens + k->tail_tokens;
+    KVC_REQUIRE(total > 0, "the cache is empty");
+    KVC_REQUIRE(v->tokens + v->tail_tokens == total, "K holds %lld tokens, V %lld", (long long)total,
+                (long long)(v->tokens + v->tail_tokens));
+    KVC_REQUIRE(k->tokens % KVC_K_VEC_PER_BLK == 0 && v->tokens % KVC_V_VEC_LEN == 0, "compressed token counts must be whole tiles");
+    KVC_REQUIRE((k->tokens == 0 || k->d_luts) && (v->tokens == 0 || v->d_luts), "decode tables are required");
+    KVC_REQUIRE((k->tail_tokens == 0 || k->d_tail_f16) && (v->tail_tokens == 0 || v->d_tail_f16), "tail pointer is NULL");
+    const KvcAttentionPlan p = kvc_attention_plan(total, v->tokens, batch, q_heads, head_dim);
+    KVC_REQUIRE(d_workspace != nullptr && ((uintptr_t)d_workspace & 255) == 0, "workspace must be 256-byte aligned");
+    KVC_REQUIRE(workspace_bytes >= p.bytes, "workspace holds %lld bytes, %lld needed", (long long)workspace_bytes, (long long)p.bytes);
+    float *scores = reinterpret_cast<float *>((char *)d_workspace + p.scores_off);
+    float *part = reinterpret_cast<float *>((char *)d_workspace + p.part_off);
+    float *ml = reinterpret_cast<float *>((char *)d_workspace + p.ml_off);
+    const int rep = (int)(q_heads / kv_heads);
+    KvcTimer timer(elapsed_ms, stream);
+    // ---- scores
+    if (k->tokens) {
+        KvcFusedExtra ex = {p.scores_stride, nullptr, 0, 1.f, nullptr};
+        if (int rc = kvc_fused(1, nullptr, 0, KVC_TREE_I8, k->d_block_infos, k->block_infos_bytes, k->d_thread_infos,
+                               k->thread_infos_bytes, k->d_encoded, k->encoded_bytes, k->d_quant_min_ints,
+                               k->d_quant_scales_f16, k->quant_mask, d_q_f16, scores, k->tokens, batch, kv_heads, q_heads,
+                               head_dim, fused_kernel_ms, stream_, (const uint32_t *)k->d_luts, (int)k->rows_per_codebook, 1,
+                               k->max_tile_bytes, k->max_stream_bytes, k->max_code_bits, &ex))
+            return rc;
+    }
+    if (k->tail_tokens) {
+        const int64_t items = k->tail_tokens * batch * kv_heads;
+        hipLaunchKernelGGL(kvc_tail_scores_kernel, dim3((unsigned)((items + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG)), dim3(KVC_WG),
+                           0, stream, reinterpret_cast<const __half *>(k->d_tail_f16), reinterpret_cast<const __half *>(d_q_f16),
+                           scores, p.scores_stride, k->tokens, k->tail_tokens, (int)batch, (int)kv_heads, rep, (int)head_dim);
+    }
+    // ---- weighted values per group
+    if (v->tokens) {
+        KvcFusedExtra ex = {0, scores, p.scores_stride, softmax_scale, ml};
+        if (int rc = kvc_fused(0, nullptr, 0, KVC_TREE_I8, v->d_block_infos, v->block_infos_bytes, v->d_thread_infos,
+                               v->thread_infos_bytes, v->d_encoded, v->encoded_bytes, v->d_quant_min_ints,
+                               v->d_quant_scales_f16, v->quant_mask, nullptr, part, v->tokens, batch, kv_heads, q_heads,
+                               head_dim, fused_kernel_ms ? fused_kernel_ms + 1 : nullptr, stream_, (const uint32_t *)v->d_luts, (int)v->rows_per_codebook, 1,
+                               v->max_tile_bytes, v->max_stream_bytes, v->max_code_bits, &ex))
+            return rc;
+    }
+    if (v->tail_tokens) {
+        const int64_t g = v->tokens / KVC_V_TOKENS;
+        hipLaunchKernelGGL(kvc_tail_values_kernel, dim3((unsigned)(batch * q_heads)), dim3(128), 0, stream,
+                           reinterpret_cast<const __half *>(v->d_tail_f16), scores, p.scores_stride, softmax_scale,
+                           part + g * batch * q_heads * head_dim, ml + g * batch * q_heads * 2, v->tokens, v->tail_tokens,
+                           (int)batch, (int)kv_heads, rep, (int)head_dim);
+    }
+    hipLaunchKernelGGL(kvc_attention_combine_kernel, dim3((unsigned)(batch * q_heads)), dim3(KVC_COMBINE_WAVES * KVC_WAVE), 0, stream, part, ml,
+                       p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+    KVC_HIP(hipGetLastError());
+    return timer.finish();
 }

@@ -223,3 +223,57 @@ def test_compressed_attention_with_wrong_or_missing_size_hints(hint):
             c.max_tile_bytes = c.max_stream_bytes = c.max_code_bits = 0
     again = CompressedAttention(kctx, vctx).attend(q)
     assert (again - good).abs().max() <= 1e-5 * good.abs().max()
+
+
+@pytest.mark.parametrize("T,D,rep,B", [(40, 128, 1, 1), (100, 128, 2, 2), (300, 64, 4, 1), (531, 96, 2, 2), (1024, 128, 8, 1)])
+def test_one_call_attention_matches_stepwise_and_fp32(T, D, rep, B):
+    """kvc_attention_decode (scores, per-group softmax, weighted values and the final merge inside the library)
+    against the same result assembled step by step with PyTorch's softmax, and against fp32 attention over the
+    dequantized cache.  Covers: nothing compressed yet, K compressed but V not, tails of different lengths."""
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant")
+    H = 2
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    att = CompressedAttention(kctx, vctx)
+    ms = []
+    out = att.attend(q, kernel_ms=ms)
+    assert len(ms) == 2 and (ms[0] > 0) == (kctx.compressed_ctx_len > 0) and (ms[1] > 0) == (vctx.compressed_ctx_len > 0)
+    again = att.attend(q)                                   # workspace reuse, no timing
+    assert torch.equal(out, again)
+    step = att.attend_stepwise(q)
+    # the stepwise path rounds the softmax weights to fp16 (the reference kernel's input format)
+    assert (out - step).abs().max() <= 2e-3 * step.abs().max()
+    kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+    s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
+    ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
+    assert (out - ref).abs().max() <= 3e-3 * ref.abs().max()
+
+
+def test_one_call_attention_grows_with_the_cache():
+    """Prefill, then decode steps that push blocks out of the tails: attention after every few steps stays
+    within tolerance of fp32 attention over what get() returns."""
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant")
+    B, H, D, rep = 1, 4, 128, 2
+    T0, steps = 200, 140
+    k, v = S.synth_k(T0 + steps, B, H, D).to(DEV), S.synth_v(T0 + steps, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k[:T0])
+    vctx.store(v[:T0])
+    att = CompressedAttention(kctx, vctx)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    for i in range(steps):
+        kctx.store(k[T0 + i:T0 + i + 1])
+        vctx.store(v[T0 + i:T0 + i + 1])
+        if i % 23 == 0 or i == steps - 1:
+            out = att.attend(q)
+            kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+            s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
+            ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
+            assert (out - ref).abs().max() <= 3e-3 * ref.abs().max(), "step %d" % i
