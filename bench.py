@@ -147,9 +147,9 @@ def codec_rates(kctx, vctx, k, v, cfg):
 # what the same counter reads for the 256 MiB kvc_calibration_copy_kernel of the same run (FETCH_SIZE x2.0,
 # WRITE_SIZE x1.0).  Source: profiles/fused_decode_attention_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2": {"kvc_fused_kernel<1, true>": int((3984.1 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, false>": int((2514.9 * 2.0 + 512.0) * 1024)},
-    "cfg3": {"kvc_fused_kernel<4, true>": int((31634.9 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, false>": int((22028.0 * 2.0 + 16384.0) * 1024)},
-    "cfg5": {"kvc_fused_kernel<1, true>": int((102890.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, false>": int((42919.1 * 2.0 + 12288.0) * 1024)},
+    "cfg2": {"kvc_fused_kernel<1, 0>": int((4041.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2696.9 * 2.0 + 528.0) * 1024)},
+    "cfg3": {"kvc_fused_kernel<4, 0>": int((31585.3 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, 3>": int((26270.6 * 2.0 + 16800.3) * 1024)},
+    "cfg5": {"kvc_fused_kernel<1, 0>": int((102429.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((46666.7 * 2.0 + 12778.7) * 1024)},
 }
 
 
