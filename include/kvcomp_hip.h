@@ -252,6 +252,20 @@ int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const void *d_scal
                 int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
                 void *d_out_f16, void *stream);
 
+/* ---- whole-tensor Huffman coder: huffman_encode (utils/huffman.py:15-95) ------------------------------
+ * kvc_h2_codes: 256 symbol counts -> per-symbol (code, length), the reference's construction (min-heap on
+ *   frequency only, first pop = left = '0'; a lone symbol gets the one-bit code '0', utils/huffman.py:42-44).
+ * kvc_h2_encode: d_sym uint8[n] (the flattened tensor, values already shifted into 0..255) -> d_bits, one byte
+ *   (0 / 1) per code bit in stream order, each code most significant bit first; *h_total_bits receives the
+ *   stream length.  d_bits == NULL only measures (the reference's callers use the length alone,
+ *   accuracy/cr_estimate.py:46-58).  d_scratch: kvc_h2_scratch_bytes(n) bytes, 8-byte aligned.  Synchronises
+ *   the stream to read the length back. */
+int kvc_h2_codes(const int64_t *h_counts256, uint32_t *h_code256, uint32_t *h_length256);
+int64_t kvc_h2_scratch_bytes(int64_t n);
+int kvc_h2_encode(const uint8_t *d_sym, int64_t n, const uint32_t *h_code256, const uint32_t *h_length256,
+                  uint8_t *d_bits, int64_t bits_cap, void *d_scratch, int64_t scratch_bytes,
+                  int64_t *h_total_bits, void *stream);
+
 /* ---- measurement aid (no counterpart in the reference) ----------------------------------------------
  * Plain device-to-device copy of `bytes` bytes (a multiple of 16) by a grid-stride kernel named
  * kvc_calibration_copy_kernel: a dispatch of exactly known HBM traffic to scale profiler counters by. */

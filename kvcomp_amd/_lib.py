@@ -50,12 +50,16 @@ _SIGNATURES = {
     "kvc_quant": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp, _vp, _vp, _vp, _vp],
     "kvc_quant_error": [_vp, _i64, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _vp],
     "kvc_calibration_copy": [_vp, _vp, _i64, _vp],
+    "kvc_h2_codes": [_i64p, _vp, _vp],
+    "kvc_h2_scratch_bytes": [_i64],
+    "kvc_h2_encode": [_vp, _i64, _vp, _vp, _vp, _i64, _vp, _i64, _i64p, _vp],
     "kvc_attention_workspace_bytes": [_i64, _i64, _i64, _i64, _i64],
     "kvc_attention_decode": [C.POINTER(CompressedDesc), C.POINTER(CompressedDesc), _vp, C.c_float, _vp, _i64, _vp,
                              _i64, _i64, _i64, _i64, _f32p, _f32p, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }
-_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_attention_workspace_bytes": _i64}
+_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_attention_workspace_bytes": _i64,
+             "kvc_h2_scratch_bytes": _i64}
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["kvc_last_error"])
 

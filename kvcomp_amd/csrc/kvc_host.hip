@@ -231,6 +231,16 @@ static int kvc_huffman_codes(const int64_t *counts, uint32_t code[256], uint32_t
     return distinct;
 }
 
+// The same construction with the lone-symbol rule of utils/huffman.py:42-44 (code '0', one bit).
+int kvc_huffman_codes_h2(const int64_t *counts, uint32_t code[256], uint32_t length[256])
+{
+    const int distinct = kvc_huffman_codes(counts, code, length);
+    if (distinct == 1)
+        for (int s = 0; s < 256; s++)
+            if (counts[s] > 0) length[s] = 1;
+    return distinct;
+}
+
 extern "C" int kvc_build_codebook_host(const int64_t *h_counts256, int tree_format, int *shift,
                                        uint8_t *h_encode_table, int64_t encode_cap, int64_t *encode_bytes,
                                        uint8_t *h_decode_tree, int64_t decode_cap, int64_t *decode_bytes)
