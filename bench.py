@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the hot path: decode attention over a Huffman-compressed KV cache on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5] [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg4|cfg5] [--no-cpu-baseline]
 
 A step is one decode-attention pass of one layer over the whole compressed cache, already resident in HBM:
 fused decompress -> q.K^T, 1/sqrt(d) + softmax, fused decompress -> p.V, partial-sum reduce.  The printed value
@@ -34,6 +34,11 @@ WORKLOADS = {
     "cfg5": dict(B=4, H=32, Hq=32, D=96, T=32768, eb_k=0.1, eb_v=0.3, dist="laplace",
                  desc="long-context decode attention, Phi-3-mini layer: batch 4, 32 heads x 96, 32768 cached tokens, Laplace + 2% x50 outliers, eb K 0.1 / V 0.3"),
 }
+# every layer of a Llama-2-7B-shaped decoder, cache path only (see run_decode_loop)
+WORKLOADS["cfg4"] = dict(layers=32, B=8, H=32, Hq=32, D=128, T=4096, eb_k=0.1, eb_v=0.2, dist="gauss",
+                         desc="decode with a compressed KV cache in all 32 layers, Llama-2-7B shape: batch 8, 32 heads x 128, "
+                              "4096-token prompt, one appended token per step, recompression every 64 (K) / 128 (V) tokens, "
+                              "eb K 0.1 / V 0.2")
 # the long-context configuration is the one the >= 70 % of HBM peak target is quoted on (32k context)
 DEFAULT_WORKLOAD = "cfg5"
 
@@ -42,20 +47,20 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def make_kv(cfg, device):
+def make_kv(cfg, device, seed_offset=0):
     """Synthetic K/V [T, B, H, D] fp16 generated on the device (seeded)."""
     import torch
     T, B, H, D = cfg["T"], cfg["B"], cfg["H"], cfg["D"]
     g = torch.Generator(device=device)
     if cfg["dist"] == "gauss":
-        g.manual_seed(1234)
+        g.manual_seed(1234 + 100 * seed_offset)
         k = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32)
         c = torch.exp(0.5 * torch.randn(H, D, generator=g, device=device, dtype=torch.float32))
         g.manual_seed(1237)
         for h in range(H):
             c[h, torch.randperm(D, generator=g, device=device)[:4]] *= 20.0
         k = (k * c).to(torch.float16)
-        g.manual_seed(1235)
+        g.manual_seed(1235 + 100 * seed_offset)
         v = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32).to(torch.float16)
     else:
         out = []
@@ -157,6 +162,73 @@ def measured_traffic(workload, kernel):
     return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
 
 
+def run_decode_loop(args):
+    """cfg4 without the model around it: every layer of a Llama-2-7B-shaped stack keeps a compressed K and V cache;
+    a step appends one new token per sequence to every layer (compressing the 64- / 128-token blocks that leave
+    the uncompressed tails) and runs decode attention over the whole cache of that layer.  Projections, MLPs and
+    sampling are not part of this path and are not run; keys, values and queries are random."""
+    import torch
+    from kvcomp_amd.ctx import KVCompCtx, KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
+    from kvcomp_amd import attention as A
+    cfg = WORKLOADS["cfg4"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L, B, H, Hq, D, T = cfg["layers"], cfg["B"], cfg["H"], cfg["Hq"], cfg["D"], cfg["T"]
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("cfg4", QuantMode.ChannelQuant, QuantMode.TokenQuant,
+                                                       64, 128, 64, 128, cfg["eb_k"], cfg["eb_v"])
+    log("[bench] %s" % cfg["desc"])
+    layers = []
+    t0 = time.perf_counter()
+    for l in range(L):
+        k, v = make_kv(cfg, dev, seed_offset=l)
+        kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
+        kctx.store(k)
+        vctx.store(v)
+        layers.append((kctx, vctx, A.CompressedAttention(kctx, vctx)))
+        del k, v
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    g = torch.Generator(device=dev).manual_seed(1236)
+    new_k = torch.randn(L, 1, B, H, D, generator=g, device=dev).to(torch.float16)
+    new_v = torch.randn(L, 1, B, H, D, generator=g, device=dev).to(torch.float16)
+    q = torch.randn(L, B, Hq, D, generator=g, device=dev).to(torch.float16)
+    out = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
+
+    def step():
+        for l, (kctx, vctx, attn) in enumerate(layers):
+            kctx.store(new_k[l])
+            vctx.store(new_v[l])
+            attn.attend(q[l], out=out)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    assert torch.isfinite(out).all()
+    comp = sum(k.compressed_bytes() + v.compressed_bytes() for k, v, _ in layers)
+    tails = sum((k.buffer.numel() + v.buffer.numel()) * 2 for k, v, _ in layers)
+    tokens = layers[0][0].ctx_len
+    raw = 2 * 2 * L * tokens * B * H * D
+    result = {
+        "metric": "decode tokens/s with a compressed KV cache in every layer (cache append + attention only)",
+        "value": round(B * args.steps / dt, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(dt / args.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8 symbols, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "cfg4: %s" % cfg["desc"], "layers": L, "context_at_end": tokens,
+                   "cache_bytes": {"compressed": comp, "fp16_tails": tails, "fp16_equivalent": raw},
+                   "compression_ratio_whole_cache": round(raw / (comp + tails), 3),
+                   "compression_ratio_compressed_part": {"k": round(layers[0][0].get_cr(), 3), "v": round(layers[0][1].get_cr(), 3)},
+                   "prefill_compress_s": round(t_prefill, 3),
+                   "not_run": "projections, MLP, norms, sampling (outside this path)"},
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,6 +236,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--eb-k", type=float, default=None, help="override the K error bound of the workload (cfg5 sweeps 0.05 / 0.1 / 0.2)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 256 MiB device copy (kvc_calibration_copy_kernel), the yardstick "
                          "for FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -177,7 +250,12 @@ def main():
     from kvcomp_amd.ctx import KVCompCtx, KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
     from kvcomp_amd import attention as A
 
-    cfg = WORKLOADS[args.workload]
+    if args.workload == "cfg4":
+        return run_decode_loop(args)
+    cfg = dict(WORKLOADS[args.workload])
+    if args.eb_k is not None:
+        cfg["desc"] = cfg["desc"].replace("eb K %g" % cfg["eb_k"], "eb K %g" % args.eb_k)
+        cfg["eb_k"] = args.eb_k
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, Hq, D, T = cfg["B"], cfg["H"], cfg["Hq"], cfg["D"], cfg["T"]

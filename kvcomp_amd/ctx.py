@@ -17,7 +17,8 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from . import kvcomp_cuda
-from .compute import QUANT_MODE_MAP, QuantMode, cut_tensor_ctx_len_0, dequant, quant, safe_cat  # noqa: F401
+from .compute import (QUANT_MODE_MAP, QuantMode, blocks_to_compress, cut_tensor_ctx_len_0, dequant, quant,  # noqa: F401
+                      safe_cat)
 
 
 class ExtractCacheConfig:
@@ -164,12 +165,36 @@ class KVCompCtx:
         self._thread_infos = _Growable()
         self._min_ints = _Growable()
         self._scales = _Growable()
-        self.buffer: Optional[torch.Tensor] = None
+        self._tail: Optional[torch.Tensor] = None      # [capacity, B, H, D]; the first _tail_len tokens are the tail
+        self._tail_len = 0
         self.max_code_bits = 0           # longest code of the codebook (0 = unknown)
         self.max_tile_bytes = 0            # largest tile payload seen so far (sizes the fused decoders' LDS staging)
         self.max_stream_bytes = 0          # longest lane stream seen so far (sizes the fused decoders' LDS rows)
         self.encode_codebook: Optional[torch.Tensor] = None
         self.decode_codebook: Optional[torch.Tensor] = None
+
+    @property
+    def buffer(self) -> Optional[torch.Tensor]:
+        """The uncompressed most recent tokens [t, B, H, D] (kvcomp_encode.py:61); a view of a preallocated area."""
+        return None if self._tail is None else self._tail[:self._tail_len]
+
+    def _tail_append(self, cache: torch.Tensor):
+        n = cache.shape[0]
+        if self._tail is None or self._tail_len + n > self._tail.shape[0]:
+            cap = max(2 * (self._tail_len + n), self.block_size + self.recent_size + 64)
+            grown = torch.empty((cap,) + tuple(cache.shape[1:]), dtype=cache.dtype, device=cache.device)
+            if self._tail_len:
+                grown[:self._tail_len] = self._tail[:self._tail_len]
+            self._tail = grown
+        self._tail[self._tail_len:self._tail_len + n] = cache
+        self._tail_len += n
+
+    def _tail_drop_front(self, n: int):
+        rest = self._tail_len - n
+        if rest > 0:
+            src = self._tail[n:self._tail_len]
+            self._tail[:rest] = src.clone() if rest > n else src       # overlapping ranges go through a copy
+        self._tail_len = rest
 
     # the reference's public tensor attributes (kvcomp_encode.py:56-61)
     encoded_data = property(lambda self: self._encoded.view)
@@ -201,9 +226,13 @@ class KVCompCtx:
             self.device = cache.device
         assert self.device == cache.device, "device mismatch"
         self.ctx_len += cache.shape[0]
-        to_compress, self.buffer = cut_tensor_ctx_len_0(self.buffer, cache, self.block_size, self.recent_size, dim=0)
-        if to_compress is None:
+        # cut_tensor_ctx_len_0 (utils/compute.py:59-72) without re-allocating the tail on every call: append in
+        # place, then the leading whole blocks that leave the tail are compressed and the rest moves to the front
+        self._tail_append(cache)
+        n_blocks = blocks_to_compress(self._tail_len, self.block_size, self.recent_size)
+        if n_blocks <= 0:
             return None
+        to_compress = self._tail[:n_blocks * self.block_size]
         blocked = to_compress.reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
         quant_ints, min_ints, quant_scale = quant(blocked, self.quant_dims, self.quant_scale_rel)
         sizes = kvcomp_cuda.calculate_buffer_size(quant_ints, self.is_k, self.head_num, self.head_dim)
@@ -224,6 +253,7 @@ class KVCompCtx:
         self._min_ints.append(min_ints)
         self._scales.append(quant_scale)
         self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
+        self._tail_drop_front(n_blocks * self.block_size)
         return quant_ints
 
     def _assert_ready(self):
@@ -258,7 +288,7 @@ class KVCompCtx:
         """kvcomp_encode.py:138-151: compressed part followed by the uncompressed tail.  (While nothing has
         been compressed yet the tail is everything; the reference asserts in that state.)"""
         if self.compressed_ctx_len == 0:
-            return self.buffer, 0.0
+            return self.buffer.clone(), 0.0
         out, t_ms = self.get_only_compressed()
         if self.buffer is not None and self.buffer.shape[0] > 0:
             out = torch.cat([out, self.buffer], dim=0)
