@@ -56,6 +56,8 @@ struct KvcFusedArgs {
     int table_words;     // LDS words reserved for the fused table (>= 1 << lbits of every codebook used)
     int pack_words;      // LDS words per wave for the packed tile payload (multiple of 4, lead words included)
     int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
+    int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
+    int double_window;   // refill 64 stream bits at a time where the vector length allows
 };
 
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
@@ -208,6 +210,93 @@ __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t las
     }
 }
 
+// The same with 64 stream bits per refill from LDS: G symbols are decoded from the low word, the window is
+// re-formed from the register pair at the bits consumed so far (fewer than 32 unless the group overflowed, which
+// `worst` reports), G more follow.  Halves the refills (address arithmetic, LDS round trip, length sums) per symbol.
+template <int G, bool CHECK, int REP>
+__device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t last_word, uint32_t &u,
+                                              uint32_t fentry_base, uint32_t mask4, int n,
+                                              const float *ops, float (&acc)[REP], uint32_t &worst)
+{
+    const float *ops_q = ops + (__lane_id() & 3);
+    for (int i = 0; i < n; i += 2 * G) {
+        uint32_t a = u >> 5;
+        a = a < last_word ? a : last_word;
+        const uint32_t w0 = stage[a], w1 = stage[a + 1], w2 = stage[a + 2];
+        constexpr int NBLK = (2 * G * REP + 3) / 4;
+        uint32_t blk[NBLK];
+#pragma unroll
+        for (int k = 0; k < NBLK; k++) blk[k] = __float_as_uint(ops_q[i * REP + 4 * k]);
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0, used1 = 0;
+        kvc_static_for<2 * G>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;
+            if (g == G) {
+                if (CHECK) used1 = es & 0xffu;
+                R = __builtin_amdgcn_alignbit(hi, lo, es);
+            }
+            const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
+            if (g != G - 1 && g != 2 * G - 1) R = __builtin_amdgcn_alignbit(R, R, e);
+            es += e;
+            const float f = __uint_as_float(e);
+            kvc_static_for<REP>([&](auto r_) {
+                constexpr int r = decltype(r_)::value;
+                constexpr int k = g * REP + r;
+                kvc_fma_quad_pick<k & 3>(acc[r], blk[k >> 2], f);
+            });
+        });
+        const uint32_t used = es & 0xffu;
+        if (CHECK) {
+            const uint32_t used2 = used - used1;
+            const uint32_t m = used1 > used2 ? used1 : used2;
+            worst = m > worst ? m : worst;
+        }
+        u += used;
+    }
+}
+
+// Two symbols per look-up.  When twice the longest code fits the index, every index decodes to exactly two
+// symbols, so the lanes stay in step (step j of the wave = elements 2j and 2j + 1) while the look-ups, window
+// shifts and length sums per symbol halve.  An entry is two words: the first symbol's fp32 pattern with the
+// length of BOTH codes in its lowest mantissa byte, then the second symbol's fp32 pattern.  Entries are
+// 8 bytes, so the window is held three bits up (look-behind of three) and "window bits & mask" is the
+// entry's byte offset.  One refill from LDS fetches 64 stream bits: two pairs are decoded from the low
+// word, the window is re-formed from the register pair at the bits consumed, two more pairs follow.
+typedef uint32_t kvc_u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) kvc_u32x2 kvc_lds_u32x2;
+
+template <int REP>
+__device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t last_word, uint32_t &u, uint32_t mask8,
+                                             uint32_t table_base, int n, const float *ops, float (&acc)[REP])
+{
+    const float *ops_q = ops + (__lane_id() & 3);
+    for (int i = 0; i < n; i += 8) {
+        uint32_t a = u >> 5;
+        a = a < last_word ? a : last_word;
+        const uint32_t w0 = stage[a], w1 = stage[a + 1], w2 = stage[a + 2];
+        constexpr int NBLK = 2 * REP;                                   // 8 symbols x REP operands, four per register
+        uint32_t blk[NBLK];
+#pragma unroll
+        for (int k = 0; k < NBLK; k++) blk[k] = __float_as_uint(ops_q[i * REP + 4 * k]);
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0;
+        kvc_static_for<4>([&](auto p_) {
+            constexpr int p = decltype(p_)::value;
+            if (p == 2) R = __builtin_amdgcn_alignbit(hi, lo, es);      // <= 24 bits consumed so far
+            const kvc_u32x2 e = *(const kvc_lds_u32x2 *)(uintptr_t)((R & mask8) | table_base);
+            if (p != 1 && p != 3) R = __builtin_amdgcn_alignbit(R, R, e.x);
+            es += e.x;
+            kvc_static_for<REP>([&](auto r_) {
+                constexpr int r = decltype(r_)::value;
+                constexpr int k0 = (2 * p) * REP + r, k1 = (2 * p + 1) * REP + r;
+                kvc_fma_quad_pick<k0 & 3>(acc[r], blk[k0 >> 2], __uint_as_float(e.x));
+                kvc_fma_quad_pick<k1 & 3>(acc[r], blk[k1 >> 2], __uint_as_float(e.y));
+            });
+        });
+        u += es & 0xffu;
+    }
+}
+
 // -- tile geometry ------------------------------------------------------------------------------------
 // KIND 0: K tile (64 tokens x head_dim channels of one (batch, head); lane = token)
 // KIND 1: V tile (128 tokens x 64 flat channels; lane = channel), head_dim a multiple of 64: one head per tile
@@ -306,7 +395,7 @@ __device__ __forceinline__ float kvc_half_bits_to_float(uint32_t bits16)
 // What the decode step needs to know about a staged tile.
 struct KvcStaged {
     bool fits;            // staged in LDS (wave-uniform); otherwise decode from global memory
-    uint32_t u0;          // fast-path start position (two bits before the first code) in the lane's LDS words
+    uint32_t u0;          // fast-path start position (`lb` bits before the first code) in the lane's LDS words
     const uint32_t *gwords;   // the lane's stream in global memory, from the aligned word holding its first byte
     uint32_t gnwords, gpos;
 };
@@ -316,7 +405,8 @@ struct KvcStaged {
 template <int REP, int KIND>
 __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int row, int col, int lane,
                                                     const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw, float *ops,
-                                                    uint32_t *pack, uint32_t *rows, float (&bias)[REP], int &sel_out)
+                                                    uint32_t *pack, uint32_t *rows, float (&bias)[REP], int &sel_out,
+                                                    uint32_t lb)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     const int D = a.head_dim;
@@ -341,11 +431,11 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
     }
     // the packed area keeps row_words spare words at its end: the copy into rows below moves the same
     // number of words for every lane, so the last lanes read past the payload
-    bool fits = KVC_PACK_LEAD + 4u * nchunks + 2u + (uint32_t)a.row_words <= (uint32_t)a.pack_words;
+    bool fits = KVC_PACK_LEAD + 4u * nchunks + 3u + (uint32_t)a.row_words <= (uint32_t)a.pack_words;
     uint32_t longest = 0;
     if (a.row_words) {
         longest = kvc_wave_max_dpp(nwords);
-        fits = fits && longest + 2u <= (uint32_t)a.row_words;
+        fits = fits && longest + 3u <= (uint32_t)a.row_words;
     }
     st.fits = fits;
     if (fits) {
@@ -443,10 +533,10 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
                 my_row[k] = wa;
                 my_row[k + 1] = wb;
             }
-            st.u0 = 32u + (first & 3u) * 8u - 2u;
+            st.u0 = 32u + (first & 3u) * 8u - lb;
             kvc_wave_sync();
         } else {
-            st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;
+            st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lb;
         }
     } else {
         st.u0 = 0;
@@ -475,14 +565,33 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
     const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
     const uint32_t lbits = lut_g[0], nlong = lut_g[2];
     const bool fast_book = nlong == 0 && (1u << lbits) <= (uint32_t)a.table_words;
-    if (fast_book)
+    // two symbols per look-up when every pair of codes fits the pair table's index
+    const uint32_t pbits = 2u * lut_g[1];
+    const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && lbits <= 7u;
+    if (pairs) {
+        // the single-symbol table goes to the (not yet used) per-wave areas, the pair table is derived from it
+        uint32_t *tmp = smem + a.table_words;
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) tmp[i] = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+        __syncthreads();
+        const uint32_t m1 = (1u << lbits) - 1u;
+        for (uint32_t idx = tid; idx < (1u << pbits); idx += KVC_WG) {
+            const uint32_t e0 = tmp[idx & m1];
+            const uint32_t e1 = tmp[(idx >> (e0 & 0xffu)) & m1];
+            smem[2 * idx] = e0 + (e1 & 0xffu);           // both lengths; they sum to at most pbits < 256
+            smem[2 * idx + 1] = e1;
+        }
+        __syncthreads();
+    } else if (fast_book) {
         for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) s_fentry[i] = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+    }
+    const uint32_t lb = pairs ? 3u : 2u;                 // look-behind bits of the window = log2(entry bytes)
     if (lane < KVC_PACK_LEAD) pack[lane] = 0;
     if (a.row_words) rows[lane * a.row_words] = 0;
     __syncthreads();
     const uint32_t mask4 = ((1u << lbits) - 1u) << 2;
     const uint32_t fgroup = lut_g[4], fcheck = lut_g[5];
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
+    const bool dwin = a.double_window != 0 && fgroup >= 4 && n % (2 * (int)fgroup) == 0;   // 64 stream bits per refill
     const uint32_t fe = (uint32_t)(uintptr_t)(kvc_lds_u32 *)s_fentry;  // 0: the table opens the dynamic LDS
 
     // this wave's tiles: T consecutive columns of one tile row
@@ -502,7 +611,7 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
     kvc_fetch_tile<REP, KIND>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
     float bias[REP];
     int sel = 0;
-    KvcStaged st = kvc_stage_tile<REP, KIND>(a, row, col0, lane, raw, ops, pack, rows, bias, sel);
+    KvcStaged st = kvc_stage_tile<REP, KIND>(a, row, col0, lane, raw, ops, pack, rows, bias, sel, lb);
     for (int it = 0; it < ntiles; it++) {
         const int col = col0 + it;
         const bool more = it + 1 < ntiles;
@@ -518,7 +627,15 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
             const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
             const uint32_t last_word = (uint32_t)(a.row_words ? a.row_words : a.pack_words) - 2u;
             uint32_t u = st.u0, worst = 0;
-            if (fgroup >= 8 && !fcheck) {
+            if (pairs) {
+                kvc_pair_dot<REP>(words, last_word - 1u, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
+            } else if (dwin && fgroup >= 8 && !fcheck) {
+                kvc_fast_dot2<8, false, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (dwin && fgroup >= 4 && fgroup < 8 && !fcheck) {
+                kvc_fast_dot2<4, false, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (dwin && fgroup >= 4 && fgroup < 8) {
+                kvc_fast_dot2<4, true, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
+            } else if (fgroup >= 8 && !fcheck) {
                 kvc_fast_dot<8, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
             } else if (fgroup >= 8) {
                 kvc_fast_dot<8, true, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
@@ -536,7 +653,7 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
             if (st.fits) {
                 const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
                 const uint32_t nw = (uint32_t)(a.row_words ? a.row_words : a.pack_words);
-                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + 2u, lut_g, n, my_ops);
+                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + lb, lut_g, n, my_ops);
             } else {
                 res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops);
             }
@@ -570,7 +687,7 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
         }
         if (more) {
             kvc_wave_sync();     // every lane is done reading this tile's LDS data
-            st = kvc_stage_tile<REP, KIND>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel);
+            st = kvc_stage_tile<REP, KIND>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel, lb);
         }
     }
 }
@@ -598,16 +715,24 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     const int force_rows = kvc_option(KVC_OPT_FUSED_ROWS);   // 0 / 1 overrides the choice below
     a.table_words = 1 << ((max_code_bits >= 1 && max_code_bits <= KVC_LUT_MAX_BITS) ? max_code_bits : KVC_LUT_MAX_BITS);
     if (a.table_words < 4) a.table_words = 4;   // keeps the per-wave areas 16-byte aligned
+    // room for the two-symbol table (8 bytes per index of 2 * longest-code bits) when the codes are short
+    const int pair_limit = kvc_option(KVC_OPT_FUSED_PAIR_BITS);
+    a.pair_bits = 0;
+    a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
+    if (max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
+        a.pair_bits = 2 * max_code_bits;
+        if (a.table_words < (2 << a.pair_bits)) a.table_words = 2 << a.pair_bits;
+    }
     const int64_t ops_words = (int64_t)slots * 128 * rep;
     const int64_t budget = (65536 / 4 - a.table_words) / KVC_WAVES_PER_WG - ops_words;   // words per wave
     const int64_t mean_tile = encoded_bytes / (tiles > 0 ? tiles : 1);
     int64_t tile_bytes = max_tile_bytes > 0 ? max_tile_bytes : 2 * mean_tile + 64;
     if (tile_bytes > KVC_MAX_TILE_BYTES) tile_bytes = KVC_MAX_TILE_BYTES;
     // lead words + the payload's chunks (it may start anywhere in its first chunk) + look-ahead
-    int64_t pack = KVC_PACK_LEAD + ((tile_bytes + 15 + 15) / 16) * 4 + 4;
+    int64_t pack = KVC_PACK_LEAD + ((tile_bytes + 15 + 15) / 16) * 4 + 4;   // three look-ahead words, rounded up
     int64_t stream_bytes = max_stream_bytes > 0 ? max_stream_bytes : 2 * mean_tile / KVC_WAVE + 4;
     // lead word + the stream's words (it may start anywhere in its first word) + look-ahead, forced odd
-    const int64_t row = ((stream_bytes + 3 + 3) / 4 + 2) | 1;
+    const int64_t row = ((stream_bytes + 3 + 3) / 4 + 3) | 1;
     const int64_t pack_rows = (pack + row + 3) / 4 * 4;      // spare words for the fixed-length copy into rows
     // Rows cost LDS space and a copy; they pay when decoding from the packed payload would line the lanes up
     // on a few banks: lane l reads about l mean-stream-lengths into the payload, so if a small multiple of
