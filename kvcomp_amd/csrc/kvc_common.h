@@ -55,7 +55,7 @@ constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2
 // ---------------------------------------------------------------------------------------------------
 int kvc_fail(int code, const char *fmt, ...);
 // Tuning knobs settable through kvc_set_option (or, before first use, KVCOMP_<NAME> in the environment).
-enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_COUNT };
+enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_COUNT };
 int kvc_option(KvcOption which);
 int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the
@@ -118,49 +118,39 @@ __device__ __forceinline__ float kvc_wave_sum(float v)
 }
 
 // Wave-wide reductions through the VALU's data-parallel lane permutes instead of LDS round trips; every lane
-// of the wave must be active.  Steps: neighbours within quads, quads within a row of 16, then the last lane
-// of a row is broadcast to the following row(s); lane 63 ends up with the total, which is read back as a scalar.
-template <class Op>
-__device__ __forceinline__ uint32_t kvc_wave_reduce_dpp(uint32_t v, Op op)
-{
-    constexpr int QUAD_SWAP1 = 0xB1, QUAD_SWAP2 = 0x4E, ROW_ROR4 = 0x124, ROW_ROR8 = 0x128, ROW_BCAST15 = 0x142,
-                  ROW_BCAST31 = 0x143;
-    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, QUAD_SWAP1, 0xf, 0xf, false));
-    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, QUAD_SWAP2, 0xf, 0xf, false));
-    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_ROR4, 0xf, 0xf, false));
-    v = op(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_ROR8, 0xf, 0xf, false));
-    // rows that receive nothing keep `old` = their own value, so they must not be combined with it: the
-    // operation is applied only where the row mask selects
-    {
-        const uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_BCAST15, 0xa, 0xf, false);
-        const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        if ((lane >> 4) & 1) v = op(v, t);
-    }
-    {
-        const uint32_t t = (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, ROW_BCAST31, 0xc, 0xf, false);
-        const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-        if (lane >= 32) v = op(v, t);
-    }
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
+// of the wave must be active.  Six steps, each one instruction whose first operand is read through the
+// permute: neighbours within quads (twice), quads within a row of 16 (rotate by 4, by 8: every lane of a row
+// then holds the row's result), then the last lane of a row is combined into the following row (rows 1 and 3),
+// and lane 31 into rows 2 and 3; lane 63 ends up with the total, which is read back as a scalar.  Rows that a
+// step does not select keep their value.  A permuted read of a register needs two idle cycles after the
+// instruction that wrote it, hence the s_nop between the steps (and in front: the input may have just been
+// written).
+#define KVC_DPP_REDUCE(op, v)                                                          \
+    asm("s_nop 1\n\t" op " %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t" \
+        "s_nop 1\n\t" op " %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t" \
+        "s_nop 1\n\t" op " %0, %0, %0 row_ror:4 row_mask:0xf bank_mask:0xf\n\t"           \
+        "s_nop 1\n\t" op " %0, %0, %0 row_ror:8 row_mask:0xf bank_mask:0xf\n\t"           \
+        "s_nop 1\n\t" op " %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"        \
+        "s_nop 1\n\t" op " %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"        \
+        "s_nop 1"                                                                          \
+        : "+v"(v))
 
 __device__ __forceinline__ float kvc_wave_sum_dpp(float v)
 {
-    return __uint_as_float(kvc_wave_reduce_dpp(__float_as_uint(v), [](uint32_t a, uint32_t b) {
-        return __float_as_uint(__uint_as_float(a) + __uint_as_float(b));
-    }));
+    KVC_DPP_REDUCE("v_add_f32_dpp", v);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __device__ __forceinline__ float kvc_wave_fmax_dpp(float v)
 {
-    return __uint_as_float(kvc_wave_reduce_dpp(__float_as_uint(v), [](uint32_t a, uint32_t b) {
-        return __float_as_uint(fmaxf(__uint_as_float(a), __uint_as_float(b)));
-    }));
+    KVC_DPP_REDUCE("v_max_f32_dpp", v);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
 __device__ __forceinline__ uint32_t kvc_wave_max_dpp(uint32_t v)
 {
-    return kvc_wave_reduce_dpp(v, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+    KVC_DPP_REDUCE("v_max_u32_dpp", v);
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
 // inclusive prefix sum over the 64 lanes of a wave

@@ -54,7 +54,9 @@ struct KvcFusedArgs {
     int64_t tokens;
     int batch, kv_heads, q_heads, head_dim;
     int table_words;     // LDS words reserved for the fused table (>= 1 << lbits of every codebook used)
-    int pack_words;      // LDS words per wave for the packed tile payload (multiple of 4, lead words included)
+    int pack_words;      // LDS words per wave reserved for the packed tile payload (multiple of 4)
+    int pack_logical;    // payload words (lead words included) that fit there; fewer than pack_words when skewed
+    int skew;            // 0, or 2: every 32 payload words are followed by a copy of the next two (see kvc_skewed)
     int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
     int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
     int double_window;   // refill 64 stream bits at a time where the vector length allows
@@ -90,6 +92,26 @@ __device__ __forceinline__ void kvc_wave_sync()
 // full bit reversal leaves stream bit k of the word at bit k
 __device__ __forceinline__ uint32_t kvc_stream_word(uint32_t raw) { return __brev(kvc_bswap(raw)); }
 
+// Skewed packed payload.  Lane l starts about l mean-stream-lengths into the payload, so when a small
+// multiple of that length is close to 32 words, every k-th lane reads the same bank at every refill.  With
+// two spare words after every 32 (holding a copy of the two words that follow, so that the three-word read
+// of a refill never has to jump), streams 32 words apart land two banks apart instead.
+//   word w of the payload lives at w + skew * (w >> 5), skew = 2 (or 0: plain layout)
+__device__ __forceinline__ uint32_t kvc_skewed(uint32_t w, uint32_t skew) { return __umul24(w >> 5, skew) + w; }
+
+// Byte address in LDS of payload word u >> 5 for a refill.  No clamp: a lane's position cannot pass its start
+// by more than 128 symbols x 10 bits, and the workgroup's LDS ends with that much slack (KVC_LDS_SLACK_WORDS),
+// so even a corrupt stream only ever reads this workgroup's own LDS.
+typedef __attribute__((address_space(3))) uint32_t kvc_lds_word;
+template <bool SKEW>
+__device__ __forceinline__ uint32_t kvc_refill_address(uint32_t stage_base, uint32_t u)
+{
+    const uint32_t a = u >> 5;
+    if (SKEW) return (a << 2) + (__umul24(u >> 10, 8u) + stage_base);     // + 2 words per 32
+    return (a << 2) + stage_base;
+}
+constexpr int KVC_LDS_SLACK_WORDS = 48;
+
 // -- slow path ----------------------------------------------------------------------------------------
 // One symbol per refill; table and long-code list in global memory; words from LDS (staged, bit-reversed)
 // or from global memory (raw, bounds-checked word by word).
@@ -101,7 +123,8 @@ struct KvcVec {
 
 template <int REP, bool GSRC>
 __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_t nwords, uint32_t pos,
-                                                  const uint32_t *__restrict__ lut_g, int n, const float *ops)
+                                                  const uint32_t *__restrict__ lut_g, int n, const float *ops,
+                                                  uint32_t skew)
 {
     const uint32_t lshift = 32u - lut_g[0], nlong = lut_g[2];
     const uint32_t *longs = lut_g + KVC_LUT_HEADER_WORDS;
@@ -113,8 +136,8 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
         const uint32_t wi = pos >> 5;
         uint32_t w0 = 0, w1 = 0;
         // either way the first stream bit of a word ends up in the most significant bit
-        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : __brev(words[wi]);
-        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : __brev(words[wi + 1]);
+        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : __brev(words[kvc_skewed(wi, skew)]);
+        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : __brev(words[kvc_skewed(wi + 1, skew)]);
         const uint32_t hi = (uint32_t)(((((uint64_t)w0) << 32 | w1) << (pos & 31u)) >> 32);
         const uint32_t e = entries[hi >> lshift];
         uint32_t len = e & 0xffu, sym = (e >> 8) & 0xffu;
@@ -171,16 +194,16 @@ __device__ __forceinline__ void kvc_fma_quad_pick(float &acc, uint32_t quad, flo
         : "v"(quad), "v"(x), "n"(J));
 }
 
-template <int G, bool CHECK, int REP>
-__device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t last_word, uint32_t &u,
+template <int G, bool CHECK, bool SKEW, int REP>
+__device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t &u,
                                              uint32_t fentry_base, uint32_t mask4, int n,
                                              const float *ops, float (&acc)[REP], uint32_t &worst)
 {
     const float *ops_q = ops + (__lane_id() & 3);
+    const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
     for (int i = 0; i < n; i += G) {
-        uint32_t a = u >> 5;
-        a = a < last_word ? a : last_word;
-        const uint32_t w0 = stage[a], w1 = stage[a + 1];
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1];
         // The group's G * REP operands, four per register: lane l holds element l & 3 of each block of four
         // and the FMA picks its operand from the right lane of the quad.  One 4-byte read per lane moves a
         // quarter of what a 16-byte broadcast read of the same four values would.
@@ -213,16 +236,16 @@ __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t las
 // The same with 64 stream bits per refill from LDS: G symbols are decoded from the low word, the window is
 // re-formed from the register pair at the bits consumed so far (fewer than 32 unless the group overflowed, which
 // `worst` reports), G more follow.  Halves the refills (address arithmetic, LDS round trip, length sums) per symbol.
-template <int G, bool CHECK, int REP>
-__device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t last_word, uint32_t &u,
+template <int G, bool CHECK, bool SKEW, int REP>
+__device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t &u,
                                               uint32_t fentry_base, uint32_t mask4, int n,
                                               const float *ops, float (&acc)[REP], uint32_t &worst)
 {
     const float *ops_q = ops + (__lane_id() & 3);
+    const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
     for (int i = 0; i < n; i += 2 * G) {
-        uint32_t a = u >> 5;
-        a = a < last_word ? a : last_word;
-        const uint32_t w0 = stage[a], w1 = stage[a + 1], w2 = stage[a + 2];
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
         constexpr int NBLK = (2 * G * REP + 3) / 4;
         uint32_t blk[NBLK];
 #pragma unroll
@@ -265,15 +288,15 @@ __device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t la
 typedef uint32_t kvc_u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) kvc_u32x2 kvc_lds_u32x2;
 
-template <int REP>
-__device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t last_word, uint32_t &u, uint32_t mask8,
+template <bool SKEW, int REP>
+__device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t &u, uint32_t mask8,
                                              uint32_t table_base, int n, const float *ops, float (&acc)[REP])
 {
     const float *ops_q = ops + (__lane_id() & 3);
+    const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
     for (int i = 0; i < n; i += 8) {
-        uint32_t a = u >> 5;
-        a = a < last_word ? a : last_word;
-        const uint32_t w0 = stage[a], w1 = stage[a + 1], w2 = stage[a + 2];
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
         constexpr int NBLK = 2 * REP;                                   // 8 symbols x REP operands, four per register
         uint32_t blk[NBLK];
 #pragma unroll
@@ -358,8 +381,10 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
         const int bh0 = (col * KVC_WAVE) / D;
         const int bh_max = a.batch * a.kv_heads - 1;
         const int64_t tk = (int64_t)row * KVC_V_TOKENS + 2 * lane;
+        const bool straddles = col * KVC_WAVE - bh0 * D + KVC_WAVE > D;   // wave-uniform
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
+            if (s == 1 && !straddles) continue;                // the second head's operands are not needed
             int bh = bh0 + s;
             bh = bh < bh_max ? bh : bh_max;                    // slot 1 is unused by a tile that ends the row
             const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
@@ -431,7 +456,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
     }
     // the packed area keeps row_words spare words at its end: the copy into rows below moves the same
     // number of words for every lane, so the last lanes read past the payload
-    bool fits = KVC_PACK_LEAD + 4u * nchunks + 3u + (uint32_t)a.row_words <= (uint32_t)a.pack_words;
+    bool fits = KVC_PACK_LEAD + 4u * nchunks + 3u + (uint32_t)a.row_words <= (uint32_t)a.pack_logical;
     uint32_t longest = 0;
     if (a.row_words) {
         longest = kvc_wave_max_dpp(nwords);
@@ -439,35 +464,35 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
     }
     st.fits = fits;
     if (fits) {
-        uint4 *p4 = reinterpret_cast<uint4 *>(pack + KVC_PACK_LEAD);
-#pragma unroll
-        for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
-            const uint32_t c = lane + 64 * j;
-            if (c < nchunks) {
-                uint4 v = raw.pay[j];
-                v.x = kvc_stream_word(v.x);
-                v.y = kvc_stream_word(v.y);
-                v.z = kvc_stream_word(v.z);
-                v.w = kvc_stream_word(v.w);
-                p4[c] = v;
-            }
-        }
-        const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
-        for (uint32_t c = lane + 64 * KVC_PRE_CHUNKS; c < nchunks; c += KVC_WAVE) {   // tiles beyond 4 KiB
-            uint4 v = g[c];
+        const uint32_t skew = (uint32_t)a.skew;
+        // chunk c holds payload words 4c .. 4c + 3 (after the lead words); chunks never straddle a run of 32
+        auto put = [&](uint32_t c, uint4 v) {
             v.x = kvc_stream_word(v.x);
             v.y = kvc_stream_word(v.y);
             v.z = kvc_stream_word(v.z);
             v.w = kvc_stream_word(v.w);
-            p4[c] = v;
+            const uint32_t w = KVC_PACK_LEAD + 4u * c;
+            uint2 *dst = reinterpret_cast<uint2 *>(pack + kvc_skewed(w, skew));     // 8-byte aligned either way
+            dst[0] = make_uint2(v.x, v.y);
+            dst[1] = make_uint2(v.z, v.w);
+            if (skew && (w & 31u) == 0u) dst[-1] = make_uint2(v.x, v.y);           // the copy that ends the previous run
+        };
+#pragma unroll
+        for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
+            const uint32_t c = lane + 64 * j;
+            if (c < nchunks) put(c, raw.pay[j]);
         }
+        const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
+        for (uint32_t c = lane + 64 * KVC_PRE_CHUNKS; c < nchunks; c += KVC_WAVE) put(c, g[c]);   // tiles beyond 4 KiB
     }
     // ---- operand table: element i of head slot s, query head r at ops[(s * 128 + i) * REP + r]
     float bias_s[SLOTS][REP];
+    const bool straddles = SLOTS == 2 && (col * KVC_WAVE) % D + KVC_WAVE > D;      // wave-uniform
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {
 #pragma unroll
         for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f;
+        if (s == 1 && !straddles) continue;                    // no lane of this tile belongs to a second head
         const bool live = KIND != 0 || 2 * lane < D;
         float wgt[REP][2];                           // the two elements' weights: q, p, or exp(score - max)
 #pragma unroll
@@ -564,14 +589,21 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
     const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
     const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
     const uint32_t lbits = lut_g[0], nlong = lut_g[2];
-    const bool fast_book = nlong == 0 && (1u << lbits) <= (uint32_t)a.table_words;
+    const bool fast_book = nlong == 0 && lbits <= (uint32_t)KVC_LUT_MAX_BITS && (1u << lbits) <= (uint32_t)a.table_words;
+    // table entries as the fast loops use them: a length beyond the index width (possible only in a table that
+    // kvc_build_lut did not write) is cut down, which bounds how far a lane's position can run (see
+    // kvc_refill_address)
+    auto fentry = [&](uint32_t i) {
+        const uint32_t e = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+        return (e & 0xffu) > lbits ? (e & ~0xffu) | lbits : e;
+    };
     // two symbols per look-up when every pair of codes fits the pair table's index
     const uint32_t pbits = 2u * lut_g[1];
     const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && lbits <= 7u;
     if (pairs) {
         // the single-symbol table goes to the (not yet used) per-wave areas, the pair table is derived from it
         uint32_t *tmp = smem + a.table_words;
-        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) tmp[i] = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) tmp[i] = fentry(i);
         __syncthreads();
         const uint32_t m1 = (1u << lbits) - 1u;
         for (uint32_t idx = tid; idx < (1u << pbits); idx += KVC_WG) {
@@ -582,7 +614,7 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
         }
         __syncthreads();
     } else if (fast_book) {
-        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) s_fentry[i] = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) s_fentry[i] = fentry(i);
     }
     const uint32_t lb = pairs ? 3u : 2u;                 // look-behind bits of the window = log2(entry bytes)
     if (lane < KVC_PACK_LEAD) pack[lane] = 0;
@@ -625,37 +657,42 @@ __global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND
         bool redo = !(fast_book && st.fits);
         if (!redo) {
             const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
-            const uint32_t last_word = (uint32_t)(a.row_words ? a.row_words : a.pack_words) - 2u;
+            const bool skew = !a.row_words && a.skew;
             uint32_t u = st.u0, worst = 0;
-            if (pairs) {
-                kvc_pair_dot<REP>(words, last_word - 1u, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
-            } else if (dwin && fgroup >= 8 && !fcheck) {
-                kvc_fast_dot2<8, false, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (dwin && fgroup >= 4 && fgroup < 8 && !fcheck) {
-                kvc_fast_dot2<4, false, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (dwin && fgroup >= 4 && fgroup < 8) {
-                kvc_fast_dot2<4, true, REP>(words, last_word - 1u, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (fgroup >= 8 && !fcheck) {
-                kvc_fast_dot<8, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (fgroup >= 8) {
-                kvc_fast_dot<8, true, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (fgroup >= 4 && !fcheck) {
-                kvc_fast_dot<4, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
-            } else if (fgroup >= 4) {
-                kvc_fast_dot<4, true, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
-            } else {
-                kvc_fast_dot<2, false, REP>(words, last_word, u, fe, mask4, n, my_ops, acc, worst);
-            }
+            auto run = [&](auto skew_) {
+                constexpr bool SK = decltype(skew_)::value;
+                if (pairs) {
+                    kvc_pair_dot<SK, REP>(words, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
+                } else if (dwin && fgroup >= 8 && !fcheck) {
+                    kvc_fast_dot2<8, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (dwin && fgroup >= 4 && fgroup < 8 && !fcheck) {
+                    kvc_fast_dot2<4, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (dwin && fgroup >= 4 && fgroup < 8) {
+                    kvc_fast_dot2<4, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (fgroup >= 8 && !fcheck) {
+                    kvc_fast_dot<8, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (fgroup >= 8) {
+                    kvc_fast_dot<8, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (fgroup >= 4 && !fcheck) {
+                    kvc_fast_dot<4, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (fgroup >= 4) {
+                    kvc_fast_dot<4, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else {
+                    kvc_fast_dot<2, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                }
+            };
+            if (skew) run(std::true_type{});
+            else run(std::false_type{});
             redo = __any(worst > 30u);
         }
         if (redo) {
             KvcVec<REP> res;
             if (st.fits) {
                 const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
-                const uint32_t nw = (uint32_t)(a.row_words ? a.row_words : a.pack_words);
-                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + lb, lut_g, n, my_ops);
+                const uint32_t nw = (uint32_t)(a.row_words ? a.row_words : a.pack_logical);
+                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + lb, lut_g, n, my_ops, a.row_words ? 0u : (uint32_t)a.skew);
             } else {
-                res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops);
+                res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops, 0u);
             }
 #pragma unroll
             for (int r = 0; r < REP; r++) acc[r] = res.v[r];
@@ -724,7 +761,7 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
         if (a.table_words < (2 << a.pair_bits)) a.table_words = 2 << a.pair_bits;
     }
     const int64_t ops_words = (int64_t)slots * 128 * rep;
-    const int64_t budget = (65536 / 4 - a.table_words) / KVC_WAVES_PER_WG - ops_words;   // words per wave
+    const int64_t budget = (65536 / 4 - a.table_words - KVC_LDS_SLACK_WORDS) / KVC_WAVES_PER_WG - ops_words;   // words per wave
     const int64_t mean_tile = encoded_bytes / (tiles > 0 ? tiles : 1);
     int64_t tile_bytes = max_tile_bytes > 0 ? max_tile_bytes : 2 * mean_tile + 64;
     if (tile_bytes > KVC_MAX_TILE_BYTES) tile_bytes = KVC_MAX_TILE_BYTES;
@@ -734,26 +771,33 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     // lead word + the stream's words (it may start anywhere in its first word) + look-ahead, forced odd
     const int64_t row = ((stream_bytes + 3 + 3) / 4 + 3) | 1;
     const int64_t pack_rows = (pack + row + 3) / 4 * 4;      // spare words for the fixed-length copy into rows
-    // Rows cost LDS space and a copy; they pay when decoding from the packed payload would line the lanes up
-    // on a few banks: lane l reads about l mean-stream-lengths into the payload, so if a small multiple of
-    // that length is close to a multiple of the 32 banks, every k-th lane hits the same bank.
+    // Decoding from the plain packed payload lines the lanes up on a few banks when a small multiple of the mean
+    // stream length is close to a multiple of the 32 banks (lane l reads about l mean-stream-lengths into the
+    // payload).  The skewed layout cures that at the cost of 1/16 more LDS and two instructions per refill;
+    // per-lane rows (an odd number of words apart) cure it too, but double the LDS a tile needs and cost a
+    // copy, so they are only used when asked for.
     const double mean_stream_words = (double)encoded_bytes / (double)(tiles > 0 ? tiles : 1) / KVC_WAVE / 4.0;
-    bool use_rows = false;
+    bool resonant = false;
     for (int k = 1; k <= 4; k++) {
         const double x = k * mean_stream_words / 32.0;
         const double dist = (x - (double)(int64_t)(x + 0.5)) * 32.0;
-        if (x >= 0.5 && dist > -1.0 && dist < 1.0) use_rows = true;
+        if (x >= 0.5 && dist > -1.0 && dist < 1.0) resonant = true;
     }
-    if (force_rows >= 0) use_rows = force_rows != 0;
-    if (use_rows && pack_rows + KVC_WAVE * row <= budget) {
+    const bool use_rows = force_rows == 1 && pack_rows + KVC_WAVE * row <= budget;
+    const int force_skew = kvc_option(KVC_OPT_FUSED_SKEW);
+    const bool use_skew = !use_rows && (force_skew >= 0 ? force_skew != 0 : resonant);
+    a.row_words = 0;
+    a.skew = 0;
+    if (use_rows) {
         a.row_words = (int)row;
         pack = pack_rows;
-    } else {
-        a.row_words = 0;
     }
-    if (pack > budget) pack = budget / 4 * 4;
-    a.pack_words = (int)pack;
-    return 4 * ((size_t)a.table_words +
+    auto physical = [&](int64_t logical) { return use_skew ? (logical + 2 * (logical >> 5) + 2 + 3) / 4 * 4 : logical; };
+    while (pack > 16 && physical(pack) > budget) pack -= 4;
+    if (use_skew) a.skew = 2;
+    a.pack_logical = (int)pack;
+    a.pack_words = (int)physical(pack);
+    return 4 * ((size_t)a.table_words + KVC_LDS_SLACK_WORDS +
                 (size_t)KVC_WAVES_PER_WG * (size_t)(ops_words + a.pack_words + KVC_WAVE * a.row_words));
 }
 

@@ -45,10 +45,11 @@ struct OptionDef {
     int fallback;
 };
 const OptionDef g_option_defs[KVC_OPT_COUNT] = {
-    {"fused_rows", "KVCOMP_FUSED_ROWS", -1},                     // -1 choose per call, 0 never, 1 whenever it fits
+    {"fused_rows", "KVCOMP_FUSED_ROWS", -1},                     // 1: per-lane rows whenever they fit; otherwise never
     {"fused_tiles_per_wave", "KVCOMP_FUSED_TILES_PER_WAVE", 0},  // 0 choose per call
     {"fused_pair_bits", "KVCOMP_FUSED_PAIR_BITS", 8},            // widest two-symbol table index; 0 = one symbol per look-up
     {"fused_double_window", "KVCOMP_FUSED_DOUBLE_WINDOW", 1},    // 64 stream bits per refill in the one-symbol loops
+    {"fused_skew", "KVCOMP_FUSED_SKEW", -1},                     // skewed payload layout: -1 choose per call, 0 never, 1 always
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;
