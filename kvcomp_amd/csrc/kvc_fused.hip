@@ -62,6 +62,9 @@ struct KvcFusedArgs {
     int double_window;   // refill 64 stream bits at a time where the vector length allows
 };
 
+#ifndef KVC_FUSED_OCC1
+#define KVC_FUSED_OCC1 5   // workgroups per CU the REP = 1 kernels are compiled for (6 spills)
+#endif
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
 
@@ -570,7 +573,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 }
 
 template <int REP, int KIND>
-__global__ void __launch_bounds__(KVC_WG, (REP <= 2 || (REP == 4 && KvcGeom<KIND>::SLOTS == 1)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 || (REP == 4 && KvcGeom<KIND>::SLOTS == 1)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
