@@ -31,10 +31,12 @@ struct KvcEncodeArgs {
     uint8_t *encoded;
     int64_t encoded_cap;
     uint32_t base_global_offset;
-    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload, [3] largest lane stream
+    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload, [3] largest lane stream;
+                               // from word KVC_ENC_STATUS_WORDS on: payload bytes of tiles 1024 j .. 1024 j + 1023
     uint32_t *idx_offset;      // {tiles, bytes}  (include/kernels.h:34-42)
 };
 
+constexpr int KVC_ENC_STATUS_WORDS = 16;            // status words in front of the per-1024-tile payload totals
 constexpr uint32_t KVC_ENC_ERR_TILE_TOO_BIG = 1u;   // a tile payload exceeds 8191 bytes
 constexpr uint32_t KVC_ENC_ERR_NO_CODE = 2u;        // a symbol without a code (length 0 or outside the table)
 constexpr uint32_t KVC_ENC_ERR_CAPACITY = 4u;       // payload does not fit encoded_cap
@@ -114,38 +116,74 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs 
     if (tid == 0) atomicMax(&a.status[3], s_longest);
 }
 
-__global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
+// Payload bytes of tiles [1024 c, 1024 c + 1024), one workgroup per c.
+__global__ void __launch_bounds__(1024) kvc_encode_chunk_sum_kernel(KvcEncodeArgs a)
 {
     __shared__ uint32_t s_wave[16];
-    __shared__ uint32_t s_carry, s_max;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) { s_carry = 0; s_max = 0; }
-    uint32_t my_max = 0;
-    __syncthreads();
-    for (int64_t base = 0; base < a.tiles; base += 1024) {
-        const int64_t tile = base + tid;
-        uint32_t bn = 0;
-        if (tile < a.tiles) bn = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile)[1] & 0xffffu;
-        my_max = bn > my_max ? bn : my_max;
-        const uint32_t incl = kvc_wave_inclusive_scan(bn, lane);
-        if (lane == KVC_WAVE - 1) s_wave[wave] = incl;
-        __syncthreads();
-        uint32_t before = s_carry;
-        for (int w = 0; w < wave; w++) before += s_wave[w];
-        if (tile < a.tiles) reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[0] = a.base_global_offset + before + incl - bn;
-        __syncthreads();
-        if (tid == 1023) s_carry = before + incl;
-        __syncthreads();
-    }
-    atomicMax(&s_max, my_max);
+    const int64_t tile = (int64_t)blockIdx.x * 1024 + tid;
+    uint32_t bn = 0;
+    if (tile < a.tiles) bn = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile)[1] & 0xffffu;
+    const uint32_t incl = kvc_wave_inclusive_scan(bn, lane);
+    if (lane == KVC_WAVE - 1) s_wave[wave] = incl;
     __syncthreads();
     if (tid == 0) {
-        const uint32_t total = s_carry;
-        a.status[0] = total;
-        a.status[2] = s_max;
-        if ((int64_t)total > a.encoded_cap) atomicOr(&a.status[1], KVC_ENC_ERR_CAPACITY);
-        a.idx_offset[0] = (uint32_t)a.tiles;
-        a.idx_offset[1] = total;
+        uint32_t total = 0;
+        for (int w = 0; w < 16; w++) total += s_wave[w];
+        a.status[KVC_ENC_STATUS_WORDS + blockIdx.x] = total;
+    }
+}
+
+// Workgroup c turns the byte_nums of tiles [1024 c, 1024 c + 1024) into offsets: what lies in front of its
+// range is the sum of the per-1024-tile totals of the kernel above, the rest is a scan of its own 1024
+// values.  No workgroup waits for another.
+__global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
+{
+    __shared__ uint32_t s_wave[16], s_before[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t *chunk_sums = a.status + KVC_ENC_STATUS_WORDS;
+    const int64_t chunks = (a.tiles + 1023) / 1024;
+    uint32_t part = 0;
+    for (int64_t j = tid; j < chunks; j += 1024) part += j < (int64_t)blockIdx.x ? chunk_sums[j] : 0u;
+    uint32_t all = 0;
+    if (blockIdx.x == 0) for (int64_t j = tid; j < chunks; j += 1024) all += chunk_sums[j];
+    const int64_t tile = (int64_t)blockIdx.x * 1024 + tid;
+    uint32_t bn = 0;
+    if (tile < a.tiles) bn = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile)[1] & 0xffffu;
+    const uint32_t incl = kvc_wave_inclusive_scan(bn, lane);
+    const uint32_t part_w = kvc_wave_inclusive_scan(part, lane);
+    uint32_t mx = bn;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)mx, off, 64);
+        mx = o > mx ? o : mx;
+    }
+    if (lane == KVC_WAVE - 1) {
+        s_wave[wave] = incl;
+        s_before[wave] = part_w;
+    }
+    if (lane == 0 && mx) atomicMax(&a.status[2], mx);
+    __syncthreads();
+    uint32_t before = a.base_global_offset;
+    for (int w = 0; w < 16; w++) {
+        before += s_before[w];
+        if (w < wave) before += s_wave[w];
+    }
+    if (tile < a.tiles) reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[0] = before + incl - bn;
+    if (blockIdx.x == 0) {
+        // the grand total, by the first workgroup
+        const uint32_t all_w = kvc_wave_inclusive_scan(all, lane);
+        __syncthreads();
+        if (lane == KVC_WAVE - 1) s_before[wave] = all_w;
+        __syncthreads();
+        if (tid == 0) {
+            uint32_t total = 0;
+            for (int w = 0; w < 16; w++) total += s_before[w];
+            a.status[0] = total;
+            if ((int64_t)total > a.encoded_cap) atomicOr(&a.status[1], KVC_ENC_ERR_CAPACITY);
+            a.idx_offset[0] = (uint32_t)a.tiles;
+            a.idx_offset[1] = total;
+        }
     }
 }
 
@@ -253,10 +291,14 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     a.base_global_offset = base_global_offset;
     a.status = reinterpret_cast<uint32_t *>(slot);
     a.idx_offset = reinterpret_cast<uint32_t *>(d_idx_offset);
-    KVC_HIP(hipMemsetAsync(slot, 0, 16, stream));
+    const int64_t chunks = (a.tiles + 1023) / 1024;
+    KVC_REQUIRE((KVC_ENC_STATUS_WORDS + chunks) * 4 <= (int64_t)KVC_WS_SLOT_BYTES, "too many tiles (%lld) for one encode call",
+                (long long)a.tiles);
+    KVC_HIP(hipMemsetAsync(slot, 0, (size_t)KVC_ENC_STATUS_WORDS * 4, stream));
     const unsigned wgs = (unsigned)((a.tiles + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
     hipLaunchKernelGGL(kvc_encode_count_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
-    hipLaunchKernelGGL(kvc_encode_scan_kernel, dim3(1), dim3(1024), 0, stream, a);
+    hipLaunchKernelGGL(kvc_encode_chunk_sum_kernel, dim3((unsigned)chunks), dim3(1024), 0, stream, a);
+    hipLaunchKernelGGL(kvc_encode_scan_kernel, dim3((unsigned)chunks), dim3(1024), 0, stream, a);
     hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     KVC_HIP(hipGetLastError());
     uint32_t h_status[4] = {0, 0, 0, 0};

@@ -335,27 +335,43 @@ extern "C" int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const v
 // ---------------------------------------------------------------------------------------------------
 // histogram
 // ---------------------------------------------------------------------------------------------------
+// One counter per (bin, lane & 31): counter (bin, c) lives in LDS bank c, so the lanes of a half wave never
+// collide on a bank, whatever the symbol distribution (KV symbols are heavily skewed: most lanes add to the
+// same one or two bins).  Only lanes l and l + 32, and the workgroup's other waves, share a counter.
 __global__ void __launch_bounds__(KVC_WG) kvc_histogram_kernel(const uint8_t *__restrict__ sym, int64_t n,
                                                                unsigned long long *__restrict__ counts)
 {
-    __shared__ uint32_t s_bins[KVC_WAVES_PER_WG][256];   // one copy per wave: fewer same-address collisions
-    const int tid = threadIdx.x, wave = tid >> 6;
-    for (int i = tid; i < KVC_WAVES_PER_WG * 256; i += KVC_WG) (&s_bins[0][0])[i] = 0;
+    __shared__ uint32_t s_bins[256 * 32];
+    const int tid = threadIdx.x, col = tid & 31;
+    for (int i = tid; i < 256 * 32; i += KVC_WG) s_bins[i] = 0;
     __syncthreads();
-    const int64_t nwords = n >> 2;
-    const uint32_t *w = reinterpret_cast<const uint32_t *>(sym);
-    for (int64_t i = (int64_t)blockIdx.x * KVC_WG + tid; i < nwords; i += (int64_t)gridDim.x * KVC_WG) {
-        const uint32_t v = w[i];
-        atomicAdd(&s_bins[wave][v & 0xffu], 1u);
-        atomicAdd(&s_bins[wave][(v >> 8) & 0xffu], 1u);
-        atomicAdd(&s_bins[wave][(v >> 16) & 0xffu], 1u);
-        atomicAdd(&s_bins[wave][v >> 24], 1u);
+    // bytes in front of the first 16-byte boundary, whole 16-byte groups, bytes after the last one
+    int64_t head = (int64_t)((16u - (uint32_t)(reinterpret_cast<uintptr_t>(sym) & 15u)) & 15u);
+    if (head > n) head = n;
+    const int64_t nquads = (n - head) >> 4;
+    const int64_t tail = n - head - (nquads << 4);
+    const uint4 *w = reinterpret_cast<const uint4 *>(sym + head);
+    auto add_word = [&](uint32_t v) {
+        atomicAdd(&s_bins[((v & 0xffu) << 5) | col], 1u);
+        atomicAdd(&s_bins[(((v >> 8) & 0xffu) << 5) | col], 1u);
+        atomicAdd(&s_bins[(((v >> 16) & 0xffu) << 5) | col], 1u);
+        atomicAdd(&s_bins[((v >> 24) << 5) | col], 1u);
+    };
+    for (int64_t i = (int64_t)blockIdx.x * KVC_WG + tid; i < nquads; i += (int64_t)gridDim.x * KVC_WG) {
+        const uint4 v = w[i];
+        add_word(v.x);
+        add_word(v.y);
+        add_word(v.z);
+        add_word(v.w);
     }
-    if (blockIdx.x == 0 && tid < (int)(n & 3)) atomicAdd(&s_bins[0][sym[(nwords << 2) + tid]], 1u);
+    if (blockIdx.x == 0) {
+        if (tid < (int)head) atomicAdd(&s_bins[((uint32_t)sym[tid] << 5) | col], 1u);
+        if (tid < (int)tail) atomicAdd(&s_bins[((uint32_t)sym[head + (nquads << 4) + tid] << 5) | col], 1u);
+    }
     __syncthreads();
     uint32_t c = 0;
 #pragma unroll
-    for (int k = 0; k < KVC_WAVES_PER_WG; k++) c += s_bins[k][tid];
+    for (int k = 0; k < 32; k++) c += s_bins[(tid << 5) | ((k + tid) & 31)];   // rotated: thread t starts at bank t
     if (c) atomicAdd(&counts[tid], (unsigned long long)c);
 }
 
@@ -363,9 +379,8 @@ extern "C" int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts,
 {
     hipStream_t stream = (hipStream_t)stream_;
     KVC_REQUIRE(n >= 0, "negative length");
-    KVC_REQUIRE(((uintptr_t)d_sym & 3) == 0, "symbol pointer must be 4-byte aligned");
     if (n == 0) return 0;
-    int64_t wgs = (n / 4 + KVC_WG * 16 - 1) / (KVC_WG * 16);   // ~64 symbols per thread, 2^32 per workgroup at most
+    int64_t wgs = (n / 16 + KVC_WG * 8 - 1) / (KVC_WG * 8);   // ~128 symbols per thread, 2^32 per workgroup at most
     if (wgs < 1) wgs = 1;
     if (wgs > 4096) wgs = 4096;
     KVC_REQUIRE(n / wgs < (1ll << 31), "input too large for 32-bit workgroup counters");
