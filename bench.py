@@ -140,11 +140,29 @@ def codec_rates(kctx, vctx, k, v, cfg):
         _, dec_ms = ctx.get_decode_quant_ints()
         _, dec_ms = ctx.get_decode_quant_ints()
         n = sym.numel()
-        out[name] = {"quantize_GBs_fp16_in": round(2 * n / ev[0].elapsed_time(ev[1]) / 1e6, 1),
+        del sym
+        # the same store as one fused call straight from fp16 (codebook known): quantize + encode, no symbol tensor
+        from kvcomp_amd.compute import dims_to_mask, mask_keepdim_shape
+        mask = dims_to_mask(ctx.quant_dims)
+        fused_ms = None
+        if m.store_fused_supported(ctx.is_k, mask, ctx.batch_size, ctx.head_num, ctx.head_dim):
+            gshape = mask_keepdim_shape(tuple(blocked.shape), mask)
+            mn = torch.empty(gshape, dtype=torch.int8, device=x.device)
+            sc = torch.empty(gshape, dtype=torch.float16, device=x.device)
+            for _ in range(2):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                m.store_fused(ctx.is_k, x, mask, ctx.quant_scale_rel, ctx.encode_codebook, mn, sc, bufs[0], bufs[1], bufs[2],
+                              bufs[3], 0)
+                e1.record()
+                torch.cuda.synchronize()
+                fused_ms = e0.elapsed_time(e1)
+            del mn, sc
+        out[name] = {"store_fused_GBs_fp16_in": round(2 * n / fused_ms / 1e6, 1) if fused_ms else None,
+                     "quantize_GBs_fp16_in": round(2 * n / ev[0].elapsed_time(ev[1]) / 1e6, 1),
                      "huffman_encode_GBs_fp16_equiv": round(2 * n / ev[2].elapsed_time(ev[3]) / 1e6, 1),
                      "huffman_encode_GBs_symbols_in": round(n / ev[2].elapsed_time(ev[3]) / 1e6, 1),
                      "huffman_decode_GBs_symbols_out": round(n / dec_ms / 1e6, 1)}
-        del sym
     return out
 
 

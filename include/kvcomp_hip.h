@@ -104,6 +104,21 @@ int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_t stride,
                          int64_t head_num, int64_t head_dim, int64_t *h_total_bytes,
                          int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream);
 
+/* ---- fused quantize + encode ---------------------------------------------------------------------------
+ * The store path of models/cache/kvcomp_encode.py:86-112 (quant, the int8 / uint8 casts, k_/v_entropy_encode)
+ * as one call straight from the fp16 cache rows: d_x_f16 is [tokens, batch, heads, head_dim] fp16, both encoder
+ * passes quantize their tile on the fly, so no symbol tensor is written or read.  Outputs are exactly those of
+ * kvc_quant followed by kvc_k_/v_entropy_encode: min_i8 / scale_f16 with the group layout of quant_mask (64-token
+ * blocks), thread_infos, block_infos, payload, idx_offset and the three host totals.
+ * Layouts: K with KVC_MASK_CHANNEL or KVC_MASK_K_BLOCK; V with KVC_MASK_V_TOKEN, or KVC_MASK_SIM_TOKEN when
+ * heads * head_dim is a multiple of 64 (kvc_store_fused_supported says which; others use the two-call path). */
+int kvc_store_fused_supported(int is_k, int quant_mask, int64_t batch, int64_t heads, int64_t head_dim);
+int kvc_store_fused(int is_k, const void *d_x_f16, int64_t tokens, int64_t batch, int64_t heads, int64_t head_dim,
+                    int quant_mask, float eb, const uint8_t *d_encode_table, int64_t encode_table_bytes,
+                    int8_t *d_min_i8, void *d_scale_f16, uint8_t *d_block_infos, uint8_t *d_thread_infos,
+                    uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
+                    int64_t *h_total_bytes, int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream);
+
 /* ---- decode: k_/v_entropy_decode_cuda_export (kernels.cu:1013-1087) -------------------------------
  * d_out uint8 [tokens, stride].  If elapsed_ms != NULL the kernel is bracketed by events, the call
  * waits for it and stores the elapsed milliseconds (the reference's return value); otherwise the call

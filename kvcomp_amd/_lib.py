@@ -33,6 +33,9 @@ _SIGNATURES = {
     "kvc_build_codebook_host": [_i64p, _int, _intp, _vp, _i64, _i64p, _vp, _i64, _i64p],
     "kvc_k_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
     "kvc_v_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
+    "kvc_store_fused_supported": [_int, _int, _i64, _i64, _i64],
+    "kvc_store_fused": [_int, _vp, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64,
+                        _u32, _i64p, _i64p, _i64p, _vp],
     "kvc_k_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_k_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,

@@ -169,8 +169,8 @@ class KVCompCacheCuda:
                cache_kwargs: Optional[Dict[str, Any]] = None) -> Tuple[torch.Tensor, torch.Tensor]:
         cos, sin = cache_kwargs['cos'], cache_kwargs['sin']
         key_states = apply_rotary_pos_emb_single(key_states, cos, sin)
-        self.k_cache_buffer[layer_idx].store(key_states.permute(2, 0, 1, 3))
-        self.v_cache_buffer[layer_idx].store(value_states.permute(2, 0, 1, 3))
+        self.k_cache_buffer[layer_idx].store(key_states.permute(2, 0, 1, 3), want_symbols=False)
+        self.v_cache_buffer[layer_idx].store(value_states.permute(2, 0, 1, 3), want_symbols=False)
         # (get() returns (tensor, milliseconds); the reference permutes the pair itself, kvcomp_encode.py:357-358)
         k_t = self.k_cache_buffer[layer_idx].get()[0].permute(1, 2, 0, 3)
         v_t = self.v_cache_buffer[layer_idx].get()[0].permute(1, 2, 0, 3)

@@ -62,6 +62,8 @@ int kvc_check_hip(hipError_t e, const char *what);
 // reference-signature entry points derive from the decode tree on every call.
 constexpr size_t KVC_WS_SLOT_BYTES = 16384;
 int kvc_workspace_slot(void **slot);
+int kvc_quant_params(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                     float eb, int8_t *d_min_i8, void *d_scale_f16, void *stream);
 int kvc_launch_build_lut(const uint8_t *d_tree, int64_t tree_bytes, int tree_format, uint32_t *d_lut,
                          int n_codebooks, int64_t tree_stride_bytes, hipStream_t stream);
 

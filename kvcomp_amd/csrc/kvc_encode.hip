@@ -15,7 +15,13 @@
 //
 // The symbols are read twice (1 B/symbol each) instead of once, which buys deterministic output
 // and no per-lane scratch area: a lane's stream may be as long as the code allows.
+//
+// kvc_store_fused runs the same count / scan / emit sequence straight from the fp16 cache: both passes
+// read the fp16 tile, quantize it (utils/compute.py:74-106, bit for bit) into an LDS tile of symbols and
+// hand each lane its vector from there, so the uint8 symbol tensor never exists in HBM (the reference
+// materialises it and several fp16 temporaries, models/cache/kvcomp_encode.py:86-98).
 #include "kvc_common.h"
+#include "kvc_quant_math.h"
 
 struct KvcEncodeArgs {
     const uint8_t *sym;        // [tokens, stride]
@@ -64,51 +70,62 @@ __device__ __forceinline__ void kvc_load_vector(const KvcEncodeArgs &a, int64_t 
     }
 }
 
+// Count pass for one tile: thread_infos, byte_num, error bits; returns the lane-stream maximum of the wave.
+__device__ __forceinline__ uint32_t kvc_count_tile(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
+                                                   const uint8_t *s_len, uint32_t *s_err)
+{
+    uint32_t bits = 0, bad = 0;
+    const int nd = a.vec_len >> 2;
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+        if (j < nd) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint32_t l = s_len[(v[j] >> (8 * k)) & 0xffu];
+                bits += l;
+                bad |= (l == 0);
+            }
+        }
+    }
+    const uint32_t bytes = (bits + 7u) >> 3;
+    const uint32_t end = kvc_wave_inclusive_scan(bytes, lane);
+    a.thread_infos[tile * KVC_WAVE + lane] = (uint16_t)((end << 3) + (bytes << 3) - bits);
+    uint32_t err = bad ? KVC_ENC_ERR_NO_CODE : 0u;
+    if (lane == KVC_WAVE - 1) {
+        if (end > (uint32_t)KVC_MAX_TILE_BYTES) err |= KVC_ENC_ERR_TILE_TOO_BIG;
+        // byte_num; the offset half of block_info is filled in by the scan kernel
+        reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[1] = end > 0xffffu ? 0xffffu : end;
+    }
+    if (err) atomicOr(s_err, err);
+    uint32_t longest = bytes;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        const uint32_t o = (uint32_t)__shfl_xor((int)longest, off, 64);
+        longest = o > longest ? o : longest;
+    }
+    return longest;
+}
+
+__device__ __forceinline__ void kvc_load_len_table(const KvcEncodeArgs &a, uint8_t *s_len, int tid)
+{
+    uint32_t len = 0;
+    if (tid < a.table_entries) len = reinterpret_cast<const uint32_t *>(a.table)[2 * tid + 1];
+    s_len[tid] = (uint8_t)(len > 32 ? 0 : len);
+}
+
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs a)
 {
     __shared__ uint8_t s_len[256];
     __shared__ uint32_t s_err, s_longest;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) { s_err = 0; s_longest = 0; }
-    {
-        uint32_t len = 0;
-        if (tid < a.table_entries) len = reinterpret_cast<const uint32_t *>(a.table)[2 * tid + 1];
-        s_len[tid] = (uint8_t)(len > 32 ? 0 : len);
-    }
+    kvc_load_len_table(a, s_len, tid);
     __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
     if (tile < a.tiles) {
         uint32_t v[32];
         kvc_load_vector(a, tile, lane, v);
-        uint32_t bits = 0, bad = 0;
-        const int nd = a.vec_len >> 2;
-#pragma unroll
-        for (int j = 0; j < 32; j++) {
-            if (j < nd) {
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint32_t l = s_len[(v[j] >> (8 * k)) & 0xffu];
-                    bits += l;
-                    bad |= (l == 0);
-                }
-            }
-        }
-        const uint32_t bytes = (bits + 7u) >> 3;
-        const uint32_t end = kvc_wave_inclusive_scan(bytes, lane);
-        a.thread_infos[tile * KVC_WAVE + lane] = (uint16_t)((end << 3) + (bytes << 3) - bits);
-        uint32_t err = bad ? KVC_ENC_ERR_NO_CODE : 0u;
-        if (lane == KVC_WAVE - 1) {
-            if (end > (uint32_t)KVC_MAX_TILE_BYTES) err |= KVC_ENC_ERR_TILE_TOO_BIG;
-            // byte_num; the offset half of block_info is filled in by the scan kernel
-            reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[1] = end > 0xffffu ? 0xffffu : end;
-        }
-        if (err) atomicOr(&s_err, err);
-        uint32_t longest = bytes;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const uint32_t o = (uint32_t)__shfl_xor((int)longest, off, 64);
-            longest = o > longest ? o : longest;
-        }
+        const uint32_t longest = kvc_count_tile(a, tile, lane, v, s_len, &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
     }
     __syncthreads();
@@ -189,6 +206,82 @@ __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
 
 constexpr int KVC_IMAGE_WORDS = (KVC_MAX_TILE_BYTES + 3 + 3) / 4 + 1;   // payload + up to 3 leading bytes
 
+// LDS traffic between the lanes of one wave needs no workgroup barrier (a wave's LDS operations complete in
+// order); this keeps the compiler from moving accesses across the hand-over.
+__device__ __forceinline__ void kvc_wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Where tile `tile` goes: ok = it fits (a tile flagged by the earlier launches is skipped, never written out of bounds).
+struct KvcEmitPlace {
+    uint32_t off, bn, head;
+    bool ok;
+};
+
+__device__ __forceinline__ KvcEmitPlace kvc_emit_place(const KvcEncodeArgs &a, int64_t tile, bool active)
+{
+    KvcEmitPlace p = {0u, 0u, 0u, false};
+    if (active) {
+        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile);
+        p.off = bi[0] - a.base_global_offset;
+        p.bn = bi[1] & 0xffffu;
+    }
+    p.ok = active && p.bn <= (uint32_t)KVC_MAX_TILE_BYTES && (int64_t)p.off + p.bn <= a.encoded_cap;
+    if (p.ok) p.head = (uint32_t)((reinterpret_cast<uintptr_t>(a.encoded) + p.off) & 3u);
+    return p;
+}
+
+// Pack this lane's vector MSB-first at its final position inside the (zeroed) LDS image of the tile payload.
+__device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
+                                                const uint2 *s_table, uint32_t *image, uint32_t head)
+{
+    const uint32_t start = lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
+    const uint32_t bitpos = (head + start) * 8u;
+    uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
+    uint64_t acc = 0;
+    const int nd = a.vec_len >> 2;
+#pragma unroll
+    for (int j = 0; j < 32; j++) {
+        if (j < nd) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const uint2 e = s_table[(v[j] >> (8 * k)) & 0xffu];
+                const uint32_t len = e.y > 32u ? 0u : e.y;
+                acc = (acc << len) | e.x;
+                nacc += len;
+                if (nacc >= 32u) {
+                    nacc -= 32u;
+                    if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
+                    w++;
+                    acc &= (1ull << nacc) - 1ull;
+                }
+            }
+        }
+    }
+    if (nacc > 0 && w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
+}
+
+// Copy the image out with aligned dword stores (bytes at the two ragged ends).
+__device__ __forceinline__ void kvc_write_image(const KvcEncodeArgs &a, const KvcEmitPlace &p, int lane, const uint32_t *image)
+{
+    uint8_t *dst = a.encoded + p.off - p.head;                 // 4-byte aligned
+    const uint32_t lo = p.head, hi = p.head + p.bn;            // valid byte range inside the image
+    const uint32_t nwords = (hi + 3u) >> 2;
+    for (uint32_t f = lane; f < nwords; f += KVC_WAVE) {
+        const uint32_t b0 = 4u * f, word = image[f];
+        if (b0 >= lo && b0 + 4u <= hi) {
+            reinterpret_cast<uint32_t *>(dst)[f] = word;
+        } else {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; k++)
+                if (b0 + k >= lo && b0 + k < hi) dst[b0 + k] = (uint8_t)(word >> (8u * k));
+        }
+    }
+}
+
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a)
 {
     __shared__ uint2 s_table[256];
@@ -196,70 +289,232 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     s_table[tid] = tid < a.table_entries ? reinterpret_cast<const uint2 *>(a.table)[tid] : make_uint2(0u, 0u);
     uint32_t *image = s_image[wave];
-    for (int i = lane; i < KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
     __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
-    const bool active = tile < a.tiles;
-    uint32_t off = 0, bn = 0, head = 0;
-    if (active) {
-        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.block_infos + 8 * tile);
-        off = bi[0] - a.base_global_offset;
-        bn = bi[1] & 0xffffu;
-    }
-    // a tile that does not fit (flagged by the earlier launches) is skipped, never written out of bounds
-    const bool ok = active && bn <= (uint32_t)KVC_MAX_TILE_BYTES && (int64_t)off + bn <= a.encoded_cap;
-    if (ok) {
-        head = (uint32_t)((reinterpret_cast<uintptr_t>(a.encoded) + off) & 3u);
-        uint32_t v[32];
-        kvc_load_vector(a, tile, lane, v);
-        const uint32_t start = lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
-        const uint32_t bitpos = (head + start) * 8u;
-        uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
-        uint64_t acc = 0;
-        const int nd = a.vec_len >> 2;
-#pragma unroll
-        for (int j = 0; j < 32; j++) {
-            if (j < nd) {
-#pragma unroll
-                for (int k = 0; k < 4; k++) {
-                    const uint2 e = s_table[(v[j] >> (8 * k)) & 0xffu];
-                    const uint32_t len = e.y > 32u ? 0u : e.y;
-                    acc = (acc << len) | e.x;
-                    nacc += len;
-                    if (nacc >= 32u) {
-                        nacc -= 32u;
-                        if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
-                        w++;
-                        acc &= (1ull << nacc) - 1ull;
-                    }
-                }
+    const KvcEmitPlace p = kvc_emit_place(a, tile, tile < a.tiles);
+    if (!p.ok) return;                                 // wave-uniform; each wave has its own image from here on
+    const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
+    for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
+    uint32_t v[32];
+    kvc_load_vector(a, tile, lane, v);
+    kvc_wave_lds_sync();
+    kvc_pack_vector(a, tile, lane, v, s_table, image, p.head);
+    kvc_wave_lds_sync();
+    kvc_write_image(a, p, lane, image);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fused quantize + encode: the front end that turns an fp16 tile into this lane's vector of symbols
+// ---------------------------------------------------------------------------------------------------
+struct KvcStoreArgs {
+    KvcEncodeArgs e;           // e.sym is unused
+    const __half *x;           // [tokens, stride] fp16
+    int B, H, D;               // stride = B * H * D
+    int mask;                  // quantization groups (KVC_MASK_*)
+    float eb;
+    int8_t *min_i8;            // per-channel K: written by the count pass; every other layout: read (written by
+    __half *scale_f16;         // the parameter pass that runs first)
+};
+
+constexpr int KVC_SYM_TILE_BYTES = 64 * (128 + 4);      // 64 vectors of up to 128 symbols, rows 4 bytes apart from a multiple of 128
+static_assert(KVC_SYM_TILE_BYTES >= KVC_IMAGE_WORDS * 4, "the payload image reuses the symbol tile");
+
+__device__ __forceinline__ KvcGroupParams kvc_stored_params(const KvcStoreArgs &a, int64_t g)
+{
+    KvcGroupParams p;
+    p.scale_h = a.scale_f16[g];
+    p.scale = __half2float(p.scale_h);
+    p.rcp = __fdiv_rn(1.0f, p.scale);
+    p.min_i = (float)a.min_i8[g];
+    p.min_h = __float2half_rn(p.min_i);
+    return p;
+}
+
+// K tile: 64 tokens x D channels of one (batch, head).  Lane l owns channels 2l and 2l + 1 while the tile is
+// quantized (each load instruction of the wave is one token's contiguous run of D halves), the symbols go
+// to LDS as [token][channel], and lane t then reads token t's vector.
+// Per-channel groups live entirely inside the tile: the count pass (PUBLISH) finds min / max itself, writes
+// the group parameters and quantizes with exactly what it wrote (the minimum as int8), the emit pass reads
+// them back, so the two passes always agree.
+template <bool PUBLISH>
+__device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t (&v)[32])
+{
+    const int64_t stride = a.e.stride;
+    const int D = a.D, RS = D + 4;
+    const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
+    const bool act = 2 * lane < D;
+    const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (act ? 2 * lane : 0);
+    auto lo = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); };
+    auto hi = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); };
+    KvcGroupParams g0, g1;
+    if (a.mask == KVC_MASK_CHANNEL) {
+        const int64_t g = row * stride + col * D + (act ? 2 * lane : 0);
+        if (PUBLISH) {
+            // two walks over the tile's rows (the second one finds them in the cache) keep the register count low
+            float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+#pragma unroll 8
+            for (int t = 0; t < KVC_WAVE; t++) {
+                const uint32_t w = *reinterpret_cast<const uint32_t *>(p + t * stride);
+                const float v0 = lo(w), v1 = hi(w);
+                mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
+                mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
             }
+            g0 = kvc_group_params(mn0, mx0, a.eb);
+            g1 = kvc_group_params(mn1, mx1, a.eb);
+            const int8_t m0 = (int8_t)(int)g0.min_i, m1 = (int8_t)(int)g1.min_i;
+            g0.min_i = (float)m0;
+            g1.min_i = (float)m1;
+            g0.min_h = __float2half_rn(g0.min_i);
+            g1.min_h = __float2half_rn(g1.min_i);
+            if (act) {
+                a.scale_f16[g] = g0.scale_h;
+                a.scale_f16[g + 1] = g1.scale_h;
+                a.min_i8[g] = m0;
+                a.min_i8[g + 1] = m1;
+            }
+        } else {
+            g0 = kvc_stored_params(a, g);
+            g1 = kvc_stored_params(a, g + 1);
         }
-        if (nacc > 0 && w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
+    } else {                                             // one pair per 64-token block (kernels.cu:771-772)
+        g0 = g1 = kvc_stored_params(a, row);
+    }
+    if (act) {
+#pragma unroll 8
+        for (int t = 0; t < KVC_WAVE; t++) {
+            const uint32_t w = *reinterpret_cast<const uint32_t *>(p + t * stride);
+            const uint32_t s2 = (uint32_t)kvc_quant_one(lo(w), g0) | ((uint32_t)kvc_quant_one(hi(w), g1) << 8);
+            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)s2;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int nd = D >> 2;
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
+}
+
+// V tile: 128 tokens x 64 flat channels.  While the tile is quantized, lane l owns channels 2 (l & 31), + 1 of
+// tokens 64 (l >> 5) .. + 63 (one load instruction = two tokens' runs of 64 halves); four tokens' symbols of a
+// channel are gathered in a register and written to LDS as one word of the [channel][token] tile, and lane c
+// then reads channel c's vector.  Group parameters are per token (KVC_MASK_V_TOKEN) or per (token, batch
+// entry) (KVC_MASK_SIM_TOKEN; the tile lies inside one batch entry); the wave first stages its 128 triples
+// {scale, 1 / scale, min} in LDS.
+__device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, float *s_par,
+                                            uint32_t (&v)[32])
+{
+    const int64_t stride = a.e.stride;
+    constexpr int RS = KVC_V_TOKENS + 4;
+    const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
+    const int pr = lane & 31, half = lane >> 5;
+    const int64_t ch = col * KVC_WAVE + 2 * pr;
+    const int64_t b = (col * KVC_WAVE) / ((int64_t)a.H * a.D);
+#pragma unroll
+    for (int k = 0; k < 2; k++) {
+        const int t = lane + 64 * k;
+        const int64_t tk = row * KVC_V_TOKENS + t;
+        const KvcGroupParams g = kvc_stored_params(a, a.mask == KVC_MASK_V_TOKEN ? tk : tk * a.B + b);
+        s_par[4 * t] = g.scale;
+        s_par[4 * t + 1] = g.rcp;
+        s_par[4 * t + 2] = g.min_i;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const __half *p = a.x + (row * KVC_V_TOKENS + 64 * half) * stride + ch;
+#pragma unroll 2
+    for (int jj = 0; jj < 16; jj++) {
+        uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const int t = 64 * half + 4 * jj + k;
+            const uint32_t raw = *reinterpret_cast<const uint32_t *>(p + (int64_t)(4 * jj + k) * stride);
+            KvcGroupParams g;
+            g.scale = s_par[4 * t];
+            g.rcp = s_par[4 * t + 1];
+            g.min_i = s_par[4 * t + 2];
+            g.min_h = __float2half_rn(g.min_i);
+            const float v0 = __half2float(__ushort_as_half((unsigned short)(raw & 0xffffu)));
+            const float v1 = __half2float(__ushort_as_half((unsigned short)(raw >> 16)));
+            w0 |= (uint32_t)kvc_quant_one(v0, g) << (8 * k);
+            w1 |= (uint32_t)kvc_quant_one(v1, g) << (8 * k);
+        }
+        *reinterpret_cast<uint32_t *>(s_sym + (2 * pr) * RS + 64 * half + 4 * jj) = w0;
+        *reinterpret_cast<uint32_t *>(s_sym + (2 * pr + 1) * RS + 64 * half + 4 * jj) = w1;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j);
+}
+
+template <bool IS_K>
+__global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
+{
+    __shared__ uint8_t s_len[256];
+    __shared__ uint32_t s_err, s_longest;
+    __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];
+    __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];   // V: {scale, 1 / scale, min, -} per token
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (tid == 0) { s_err = 0; s_longest = 0; }
+    kvc_load_len_table(a.e, s_len, tid);
+    __syncthreads();
+    const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    if (tile < a.e.tiles) {
+        uint32_t v[32];
+        if (IS_K) kvc_front_k<true>(a, tile, lane, s_sym[wave], v);
+        else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+        const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len, &s_err);
+        if (lane == 0) atomicMax(&s_longest, longest);
     }
     __syncthreads();
-    if (ok) {
-        uint8_t *dst = a.encoded + off - head;                 // 4-byte aligned
-        const uint32_t lo = head, hi = head + bn;              // valid byte range inside the image
-        const uint32_t nwords = (hi + 3u) >> 2;
-        for (uint32_t f = lane; f < nwords; f += KVC_WAVE) {
-            const uint32_t b0 = 4u * f, word = image[f];
-            if (b0 >= lo && b0 + 4u <= hi) {
-                reinterpret_cast<uint32_t *>(dst)[f] = word;
-            } else {
-#pragma unroll
-                for (uint32_t k = 0; k < 4; k++)
-                    if (b0 + k >= lo && b0 + k < hi) dst[b0 + k] = (uint8_t)(word >> (8u * k));
-            }
-        }
-    }
+    if (tid == 0 && s_err) atomicOr(&a.e.status[1], s_err);
+    if (tid == 0) atomicMax(&a.e.status[3], s_longest);
 }
+
+template <bool IS_K>
+__global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
+{
+    __shared__ uint2 s_table[256];
+    __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];   // symbols first, then the payload image
+    __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    s_table[tid] = tid < a.e.table_entries ? reinterpret_cast<const uint2 *>(a.e.table)[tid] : make_uint2(0u, 0u);
+    __syncthreads();
+    const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    const KvcEmitPlace p = kvc_emit_place(a.e, tile, tile < a.e.tiles);
+    if (!p.ok) return;                                 // wave-uniform; nothing below involves another wave
+    uint32_t *image = reinterpret_cast<uint32_t *>(s_sym[wave]);
+    uint32_t v[32];
+    if (IS_K) kvc_front_k<false>(a, tile, lane, s_sym[wave], v);
+    else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+    kvc_wave_lds_sync();                               // every lane holds its vector: the tile can be overwritten
+    const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
+    for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
+    kvc_wave_lds_sync();
+    kvc_pack_vector(a.e, tile, lane, v, s_table, image, p.head);
+    kvc_wave_lds_sync();
+    kvc_write_image(a.e, p, lane, image);
+}
+
+// What the fused path adds to an encode call: the fp16 source and how to quantize it.
+struct KvcStoreSource {
+    const void *x_f16;
+    int64_t B, H;
+    int mask;
+    float eb;
+    int8_t *min_i8;
+    void *scale_f16;
+};
 
 static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, int64_t stride,
                               const uint8_t *d_encode_table, int64_t encode_table_bytes, uint8_t *d_block_infos,
                               uint8_t *d_thread_infos, uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
                               uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes,
-                              int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream_)
+                              int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream_,
+                              const KvcStoreSource *src = nullptr)
 {
     hipStream_t stream = (hipStream_t)stream_;
     int64_t sizes[4];
@@ -272,6 +527,7 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     KVC_REQUIRE(((uintptr_t)d_encode_table & 7) == 0 && ((uintptr_t)d_block_infos & 3) == 0 &&
                 ((uintptr_t)d_thread_infos & 1) == 0 && ((uintptr_t)d_idx_offset & 3) == 0 && ((uintptr_t)d_sym & 3) == 0,
                 "encode buffers are misaligned");
+    KVC_REQUIRE(src != nullptr || d_sym != nullptr, "symbol pointer is NULL");
     KVC_REQUIRE(stride % 4 == 0, "stride must be a multiple of 4");
     void *slot;
     if (int rc = kvc_workspace_slot(&slot)) return rc;
@@ -296,10 +552,26 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
                 (long long)a.tiles);
     KVC_HIP(hipMemsetAsync(slot, 0, (size_t)KVC_ENC_STATUS_WORDS * 4, stream));
     const unsigned wgs = (unsigned)((a.tiles + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
-    hipLaunchKernelGGL(kvc_encode_count_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
+    KvcStoreArgs sa;
+    if (src) {
+        sa.e = a;
+        sa.x = reinterpret_cast<const __half *>(src->x_f16);
+        sa.B = (int)src->B;
+        sa.H = (int)src->H;
+        sa.D = (int)head_dim;
+        sa.mask = src->mask;
+        sa.eb = src->eb;
+        sa.min_i8 = src->min_i8;
+        sa.scale_f16 = reinterpret_cast<__half *>(src->scale_f16);
+    }
+    if (!src) hipLaunchKernelGGL(kvc_encode_count_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
+    else if (is_k) hipLaunchKernelGGL(kvc_store_count_kernel<true>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
+    else hipLaunchKernelGGL(kvc_store_count_kernel<false>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
     hipLaunchKernelGGL(kvc_encode_chunk_sum_kernel, dim3((unsigned)chunks), dim3(1024), 0, stream, a);
     hipLaunchKernelGGL(kvc_encode_scan_kernel, dim3((unsigned)chunks), dim3(1024), 0, stream, a);
-    hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
+    if (!src) hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
+    else if (is_k) hipLaunchKernelGGL(kvc_store_emit_kernel<true>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
+    else hipLaunchKernelGGL(kvc_store_emit_kernel<false>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
     KVC_HIP(hipGetLastError());
     uint32_t h_status[4] = {0, 0, 0, 0};
     KVC_HIP(hipMemcpyAsync(h_status, slot, 16, hipMemcpyDeviceToHost, stream));
@@ -337,4 +609,46 @@ extern "C" int kvc_v_entropy_encode(const uint8_t *d_sym, int64_t tokens, int64_
     return kvc_entropy_encode(0, d_sym, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
                               d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
                               h_max_tile_bytes, h_max_stream_bytes, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// fused quantize + encode (no counterpart in the reference, which quantizes with ~8 fp16 tensor ops into a
+// uint8 tensor and then encodes that: models/cache/kvcomp_encode.py:86-112)
+// ---------------------------------------------------------------------------------------------------
+extern "C" int kvc_store_fused_supported(int is_k, int quant_mask, int64_t batch, int64_t heads, int64_t head_dim)
+{
+    if (batch <= 0 || heads <= 0 || head_dim <= 0 || head_dim > 128 || head_dim % 8 != 0) return 0;
+    if (is_k) return quant_mask == KVC_MASK_CHANNEL || quant_mask == KVC_MASK_K_BLOCK;
+    if (quant_mask == KVC_MASK_V_TOKEN) return 1;
+    return quant_mask == KVC_MASK_SIM_TOKEN && (heads * head_dim) % KVC_V_VEC_PER_BLK == 0;
+}
+
+extern "C" int kvc_store_fused(int is_k, const void *d_x_f16, int64_t tokens, int64_t batch, int64_t heads, int64_t head_dim,
+                               int quant_mask, float eb, const uint8_t *d_encode_table, int64_t encode_table_bytes,
+                               int8_t *d_min_i8, void *d_scale_f16, uint8_t *d_block_infos, uint8_t *d_thread_infos,
+                               uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
+                               int64_t *h_total_bytes, int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream)
+{
+    KVC_REQUIRE(kvc_store_fused_supported(is_k, quant_mask, batch, heads, head_dim),
+                "fused store: unsupported layout (is_k %d, groups 0x%x, %lld heads x %lld)", is_k, quant_mask,
+                (long long)heads, (long long)head_dim);
+    KVC_REQUIRE(d_x_f16 != nullptr && d_min_i8 != nullptr && d_scale_f16 != nullptr, "NULL argument");
+    KVC_REQUIRE(((uintptr_t)d_x_f16 & 3) == 0 && ((uintptr_t)d_scale_f16 & 1) == 0, "fp16 buffers are misaligned");
+    KVC_REQUIRE(eb > 0.f, "error bound must be positive");
+    const int64_t stride = batch * heads * head_dim;
+    const int64_t bs = KVC_K_VEC_PER_BLK;                 // quantization block = 64 tokens in every supported layout
+    KVC_REQUIRE(tokens >= 0 && tokens % (is_k ? KVC_K_VEC_PER_BLK : KVC_V_VEC_LEN) == 0, "token count must be whole tiles");
+    if (tokens == 0) {
+        if (h_total_bytes) *h_total_bytes = 0;
+        return 0;
+    }
+    // every layout but per-channel K needs its group parameters before any tile can be quantized
+    if (quant_mask != KVC_MASK_CHANNEL) {
+        if (int rc = kvc_quant_params(d_x_f16, tokens / bs, bs, batch, heads, head_dim, quant_mask, eb, d_min_i8, d_scale_f16, stream))
+            return rc;
+    }
+    KvcStoreSource src = {d_x_f16, batch, heads, quant_mask, eb, d_min_i8, d_scale_f16};
+    return kvc_entropy_encode(is_k, nullptr, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
+                              d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
+                              h_max_tile_bytes, h_max_stream_bytes, stream, &src);
 }

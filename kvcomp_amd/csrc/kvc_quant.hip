@@ -12,48 +12,7 @@
 // the exact fp16 inputs followed by one rounding to fp16.  The device code spells out exactly that
 // chain; the fp32 division is IEEE (correctly rounded) and fp16/fp32 subnormals are kept.
 #include "kvc_common.h"
-
-// ---------------------------------------------------------------------------------------------------
-// scalar pieces of the reference arithmetic
-// ---------------------------------------------------------------------------------------------------
-struct KvcGroupParams {
-    float scale;     // exact value of the fp16 scale
-    float min_i;     // exact value of the fp16 rounded min / scale
-    __half scale_h, min_h;
-};
-
-__device__ __forceinline__ KvcGroupParams kvc_group_params(float mn, float mx, float eb)
-{
-    KvcGroupParams g;
-    const __half range = __float2half_rn(mx - mn);                          // (max_ - min_)
-    g.scale_h = __float2half_rn(__half2float(range) * eb);                  // * quant_scale_rel
-    g.scale = __half2float(g.scale_h);
-    const __half mq = __float2half_rn(__fdiv_rn(mn, g.scale));              // min_ / quant_scale
-    g.min_h = __float2half_rn(rintf(__half2float(mq)));                     // .round_()
-    g.min_i = __half2float(g.min_h);
-    return g;
-}
-
-__device__ __forceinline__ __half kvc_quant_one_f16(float x, const KvcGroupParams &g)
-{
-    const __half q = __float2half_rn(__fdiv_rn(x, g.scale));                // tensor / quant_scale
-    const float qi = __half2float(__float2half_rn(rintf(__half2float(q)))); // .round_()
-    return __float2half_rn(qi - g.min_i);                                   // quant_ints - min_ints
-}
-
-__device__ __forceinline__ uint8_t kvc_quant_one(float x, const KvcGroupParams &g)
-{
-    return (uint8_t)(int)__half2float(kvc_quant_one_f16(x, g));             // .to(torch.uint8)
-}
-
-// The value the simulated-quantization path keeps (utils/compute.py:130): (quant_int + min_quant) * quant_scale,
-// two fp16 tensor ops on the un-cast fp16 symbol and minimum.
-__device__ __forceinline__ __half kvc_quant_error_one(float x, const KvcGroupParams &g)
-{
-    const __half s = kvc_quant_one_f16(x, g);
-    const __half sum = __float2half_rn(__half2float(s) + g.min_i);
-    return __float2half_rn(__half2float(sum) * g.scale);
-}
+#include "kvc_quant_math.h"
 
 __device__ __forceinline__ float kvc_wave_min(float v)
 {
@@ -133,6 +92,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_kernel(KvcQuantArgs 
     const int64_t g = nb * stride + c;
     kvc_quant_publish(a, g, g0);
     kvc_quant_publish(a, g + 1, g1);
+    if (!a.sym && !a.xhat) return;                        // parameters only
     const int64_t base = nb * a.BS * stride + c;
     for (int64_t t = 0; t < a.BS; t++) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + t * stride);
@@ -159,6 +119,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, i
     mx = kvc_wave_max(mx);
     const KvcGroupParams gp = kvc_group_params(mn, mx, a.eb);
     if (lane == 0) kvc_quant_publish(a, g, gp);
+    if (!a.sym && !a.xhat) return;                        // parameters only
     for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
         kvc_quant_store2(a, g * R + i, __low2float(v), __high2float(v), gp, gp);
@@ -212,6 +173,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_block_apply_kernel(KvcQuantA
     // the first row of a group also publishes the group's metadata
     const bool first = a.mask == KVC_MASK_K_BLOCK ? (row % a.BS == 0) : ((row / a.B) % a.BS == 0);
     if (first && lane == 0) kvc_quant_publish(a, g, gp);
+    if (!a.sym && !a.xhat) return;                        // parameters only
     const __half *p = a.x + row * R;
     for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
         const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
@@ -284,6 +246,14 @@ extern "C" int kvc_quant(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B,
     KVC_REQUIRE(d_sym != nullptr && d_min_i8 != nullptr && d_scale_f16 != nullptr, "output pointer is NULL");
     return kvc_quant_launch(d_x_f16, NB, BS, B, H, D, quant_mask, eb, d_sym, d_min_i8, d_scale_f16, d_min_f16, nullptr,
                             d_counts, stream);
+}
+
+// group parameters (min_i8, scale) without symbols: the first pass of the fused quantize + encode path
+int kvc_quant_params(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
+                     float eb, int8_t *d_min_i8, void *d_scale_f16, void *stream)
+{
+    return kvc_quant_launch(d_x_f16, NB, BS, B, H, D, quant_mask, eb, nullptr, d_min_i8, d_scale_f16, nullptr, nullptr,
+                            nullptr, stream);
 }
 
 extern "C" int kvc_quant_error(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,

@@ -17,8 +17,8 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from . import kvcomp_cuda
-from .compute import (QUANT_MODE_MAP, QuantMode, blocks_to_compress, cut_tensor_ctx_len_0, dequant, quant,  # noqa: F401
-                      safe_cat)
+from .compute import (QUANT_MODE_MAP, QuantMode, blocks_to_compress, cut_tensor_ctx_len_0, dequant, dims_to_mask,  # noqa: F401
+                      mask_keepdim_shape, quant, safe_cat)
 
 
 class ExtractCacheConfig:
@@ -218,9 +218,14 @@ class KVCompCtx:
         return (KVCompCtx.block_infos_buffer[dev], KVCompCtx.thread_infos_buffer[dev],
                 KVCompCtx.idx_offset_buffer[dev], KVCompCtx.pre_alloc_compressed_data_buffer[dev])
 
-    def store(self, cache: torch.Tensor):
+    # With a codebook in place, whole blocks can go from fp16 to payload in one library call that never
+    # materialises the symbols; callers that do not look at store()'s return value ask for it.
+    fused_store = True
+
+    def store(self, cache: torch.Tensor, want_symbols: bool = True):
         """kvcomp_encode.py:69-136: append [T_new, B, H, D]; compress the whole blocks that leave the tail.
-        Returns the uint8 symbols that were compressed (None if nothing left the tail)."""
+        Returns the uint8 symbols that were compressed (None if nothing left the tail, or if want_symbols is
+        False and the fused quantize + encode path ran)."""
         self._check(cache)
         if self.device is None:
             self.device = cache.device
@@ -233,6 +238,12 @@ class KVCompCtx:
         if n_blocks <= 0:
             return None
         to_compress = self._tail[:n_blocks * self.block_size]
+        mask = dims_to_mask(self.quant_dims)
+        if (not want_symbols and KVCompCtx.fused_store and self.encode_codebook is not None
+                and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
+            self._store_fused(to_compress, mask)
+            self._tail_drop_front(n_blocks * self.block_size)
+            return None
         blocked = to_compress.reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
         quant_ints, min_ints, quant_scale = quant(blocked, self.quant_dims, self.quant_scale_rel)
         sizes = kvcomp_cuda.calculate_buffer_size(quant_ints, self.is_k, self.head_num, self.head_dim)
@@ -255,6 +266,29 @@ class KVCompCtx:
         self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
         self._tail_drop_front(n_blocks * self.block_size)
         return quant_ints
+
+    def _store_fused(self, to_compress: torch.Tensor, mask: int):
+        """fp16 rows -> payload + metadata in one call (kvc_store_fused); same outputs as the two-step path."""
+        T = to_compress.shape[0]
+        nb = T // self.block_size
+        gshape = mask_keepdim_shape((nb, self.block_size, self.batch_size, self.head_num, self.head_dim), mask)
+        min_ints = torch.empty(gshape, dtype=torch.int8, device=self.device)
+        quant_scale = torch.empty(gshape, dtype=torch.float16, device=self.device)
+        sizes = kvcomp_cuda.buffer_sizes(T, self.batch_size * self.head_num * self.head_dim, self.is_k, self.head_num,
+                                         self.head_dim)
+        KVCompCtx.buffer_ctx_len[self.device] = T
+        bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
+        encoded_, block_infos_, vec_infos_ = kvcomp_cuda.store_fused(
+            self.is_k, to_compress, mask, self.quant_scale_rel, self.encode_codebook, min_ints, quant_scale, bi_buf, ti_buf,
+            idx_buf, payload_buf, self._encoded.used)
+        self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
+        self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
+        self._encoded.append(encoded_)
+        self._block_infos.append(block_infos_)
+        self._thread_infos.append(vec_infos_)
+        self._min_ints.append(min_ints)
+        self._scales.append(quant_scale)
+        self.compressed_ctx_len += T
 
     def _assert_ready(self):
         assert self.quant_min_ints is not None, "quant_min_ints is None"

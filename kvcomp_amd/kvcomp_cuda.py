@@ -127,6 +127,48 @@ def _entropy_encode(is_k, input, encode_code_book, block_infos, thread_infos, id
     return encoded_data[:total.value], block_infos[:sizes[0]], thread_infos[:sizes[1]]
 
 
+def buffer_sizes(tokens: int, stride: int, is_k: bool, head_num: int, head_dim: int) -> Tuple[int, int, int, int]:
+    """calculate_buffer_size (src/kernels.cu:893-917) from the geometry alone."""
+    out4 = (C.c_int64 * 4)()
+    check(_lib.lib().kvc_calculate_buffer_size(tokens, stride, int(is_k), head_num, head_dim, out4))
+    return tuple(int(v) for v in out4)
+
+
+def store_fused_supported(is_k: bool, quant_mask: int, batch: int, head_num: int, head_dim: int) -> bool:
+    return bool(_lib.lib().kvc_store_fused_supported(int(is_k), quant_mask, batch, head_num, head_dim))
+
+
+def store_fused(is_k: bool, cache: torch.Tensor, quant_mask: int, quant_scale_rel: float, encode_code_book, min_ints, scales,
+                block_infos, thread_infos, idx_offset, encoded_data, base_global_offset: int):
+    """Quantize + Huffman-encode fp16 cache rows [T, B, H, D] in one library call (no counterpart in the reference,
+    which runs quant and the encoder separately: models/cache/kvcomp_encode.py:86-112).  min_ints (int8) and scales
+    (fp16) receive the group parameters; returns views (payload, block_infos, thread_infos) like the encoders."""
+    _require(cache.is_cuda and cache.dtype == torch.float16 and cache.dim() == 4 and cache.is_contiguous(),
+             "cache must be a contiguous device float16 tensor [T, B, H, D]")
+    for t, n in ((encode_code_book, "encode_code_book"), (block_infos, "block_infos"), (thread_infos, "thread_infos"),
+                 (idx_offset, "idx_offset"), (encoded_data, "encoded_data")):
+        _dev_u8(t, n)
+    T, B, H, D = cache.shape
+    sizes = buffer_sizes(T, B * H * D, is_k, H, D)
+    _require(block_infos.numel() >= sizes[0], "block_infos buffer too small")
+    _require(thread_infos.numel() >= sizes[1], "thread_infos buffer too small")
+    _require(idx_offset.numel() >= sizes[2], "idx_offset buffer too small")
+    groups = _lib.lib().kvc_quant_groups(T // 64, 64, B, H, D, quant_mask)
+    _require(min_ints.dtype == torch.int8 and min_ints.numel() >= groups and min_ints.is_cuda, "min_ints: int8 device tensor of the group count")
+    _require(scales.dtype == torch.float16 and scales.numel() >= groups and scales.is_cuda, "scales: fp16 device tensor of the group count")
+    total, max_tile, max_stream = C.c_int64(0), C.c_int64(0), C.c_int64(0)
+    with torch.cuda.device(cache.device):
+        check(_lib.lib().kvc_store_fused(int(is_k), _ptr(cache), T, B, H, D, quant_mask, float(quant_scale_rel),
+                                         _ptr(encode_code_book), encode_code_book.numel(), _ptr(min_ints), _ptr(scales),
+                                         _ptr(block_infos), _ptr(thread_infos), _ptr(idx_offset), _ptr(encoded_data),
+                                         encoded_data.numel(), int(base_global_offset) & 0xFFFFFFFF, C.byref(total),
+                                         C.byref(max_tile), C.byref(max_stream), _stream(cache)))
+    global last_encode_max_tile_bytes, last_encode_max_stream_bytes
+    last_encode_max_tile_bytes = int(max_tile.value)
+    last_encode_max_stream_bytes = int(max_stream.value)
+    return encoded_data[:total.value], block_infos[:sizes[0]], thread_infos[:sizes[1]]
+
+
 def k_entropy_encode_cuda_export(input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
                                  base_global_offset: int, head_num: int, head_dim: int):
     """src/kernels.cu:919-966.  Returns views (payload, block_infos, thread_infos) of the caller's scratch."""
