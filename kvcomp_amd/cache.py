@@ -164,6 +164,8 @@ class KVCompCacheCuda:
         self.head_dim = head_dim
         self.k_cache_buffer = [KVCompCtx(True, batch_size, head_num, head_dim, cfg.k_quant_scale_rel) for _ in range(layer_num)]
         self.v_cache_buffer = [KVCompCtx(False, batch_size, head_num, head_dim, cfg.v_quant_scale_rel) for _ in range(layer_num)]
+        for ctx in self.k_cache_buffer + self.v_cache_buffer:
+            ctx.codebook_smoothing = True        # tokens generated later may quantize to symbols the prompt never produced
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[Dict[str, Any]] = None) -> Tuple[torch.Tensor, torch.Tensor]:

@@ -12,6 +12,7 @@ get_only_compressed, get_decode_quant_ints, mat_vec_mul, build_codebook, get_cr)
   * batch > 1 and per-channel K (QuantMode.ChannelQuant) are accepted.
 """
 import ast
+import math
 from typing import Dict, List, Optional, Tuple
 
 import torch
@@ -250,8 +251,11 @@ class KVCompCtx:
         KVCompCtx.buffer_ctx_len[self.device] = to_compress.shape[0]
         bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
         if self.encode_codebook is None:     # first stored chunk defines the codebook (kvcomp_encode.py:99-103)
-            shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
-            assert shift == 0, "shift must be 0"
+            if self.codebook_smoothing:
+                enc, dec = self._smoothed_codebook(quant_ints)
+            else:
+                shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
+                assert shift == 0, "shift must be 0"
             self._set_codebook(enc, dec)
         fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
         encoded_, block_infos_, vec_infos_ = fn(quant_ints, self.encode_codebook, bi_buf, ti_buf, idx_buf, payload_buf,
@@ -266,6 +270,20 @@ class KVCompCtx:
         self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
         self._tail_drop_front(n_blocks * self.block_size)
         return quant_ints
+
+    # The reference derives the one codebook of a stream from its first stored chunk alone, so a symbol that first
+    # shows up later has no code (its encoder then emits nothing for it and the stream is corrupt; here the
+    # encoder reports an error).  With smoothing, every symbol the error bound allows counts once more than it
+    # occurs, so all of them get a code; the codebook then differs from the reference's for the same chunk.
+    codebook_smoothing = False
+
+    def _smoothed_codebook(self, quant_ints: torch.Tensor):
+        n_sym = min(256, int(math.ceil(1.0 / self.quant_scale_rel)) + 3)      # symbols 0 .. ceil(1 / eb) + 2
+        counts = kvcomp_cuda.symbol_counts([quant_ints])
+        counts[:n_sym] += 1
+        shift, enc, dec = kvcomp_cuda.build_codebook_from_counts(counts)
+        assert shift == 0, "shift must be 0"
+        return enc, dec
 
     def _store_fused(self, to_compress: torch.Tensor, mask: int):
         """fp16 rows -> payload + metadata in one call (kvc_store_fused); same outputs as the two-step path."""

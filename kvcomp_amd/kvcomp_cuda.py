@@ -76,6 +76,11 @@ def build_codebook(input_tensors: List[torch.Tensor], tree_format: int = TREE_I8
     """src/huffman.cpp:99-157: histogram of all inputs -> (shift, encode table, decode tree) as CPU uint8
     tensors.  The histogram runs on the device the inputs live on (one 2 KiB copy back, where the
     reference issues 256 .item() reads, huffman.cpp:42)."""
+    return build_codebook_from_counts(symbol_counts(input_tensors), tree_format)
+
+
+def symbol_counts(input_tensors: List[torch.Tensor]) -> torch.Tensor:
+    """256-bin histogram of device uint8 tensors (torch::bincount in src/huffman.cpp:105-109), as a CPU int64 tensor."""
     _require(len(input_tensors) > 0, "input_tensors must not be empty")
     dev = input_tensors[0].device
     for t in input_tensors:
@@ -87,8 +92,7 @@ def build_codebook(input_tensors: List[torch.Tensor], tree_format: int = TREE_I8
         for t in input_tensors:
             t = t.contiguous()
             check(L.kvc_histogram(_ptr(t), t.numel(), _ptr(counts), _stream(t)))
-        h_counts = counts.cpu()
-    return build_codebook_from_counts(h_counts, tree_format)
+        return counts.cpu()
 
 
 def build_codebook_from_counts(counts: torch.Tensor, tree_format: int = TREE_I8):
