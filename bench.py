@@ -139,6 +139,8 @@ def codec_rates(kctx, vctx, k, v, cfg):
         torch.cuda.synchronize()
         _, dec_ms = ctx.get_decode_quant_ints()
         _, dec_ms = ctx.get_decode_quant_ints()
+        _, deq_ms = ctx.get_only_compressed()               # decode + dequantize in one kernel: fp16 out
+        _, deq_ms = ctx.get_only_compressed()
         n = sym.numel()
         del sym
         # the same store as one fused call straight from fp16 (codebook known): quantize + encode, no symbol tensor
@@ -162,7 +164,8 @@ def codec_rates(kctx, vctx, k, v, cfg):
                      "quantize_GBs_fp16_in": round(2 * n / ev[0].elapsed_time(ev[1]) / 1e6, 1),
                      "huffman_encode_GBs_fp16_equiv": round(2 * n / ev[2].elapsed_time(ev[3]) / 1e6, 1),
                      "huffman_encode_GBs_symbols_in": round(n / ev[2].elapsed_time(ev[3]) / 1e6, 1),
-                     "huffman_decode_GBs_symbols_out": round(n / dec_ms / 1e6, 1)}
+                     "huffman_decode_GBs_symbols_out": round(n / dec_ms / 1e6, 1),
+                     "decode_dequant_GBs_fp16_out": round(2 * n / deq_ms / 1e6, 1)}
     return out
 
 

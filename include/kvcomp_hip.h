@@ -136,6 +136,19 @@ int kvc_v_entropy_decode(const uint8_t *d_encoded, int64_t encoded_bytes,
                          uint8_t *d_out, int64_t tokens, int64_t stride,
                          int64_t head_num, int64_t head_dim, float *elapsed_ms, void *stream);
 
+/* ---- decode + dequantize: KVCompCtx.get_only_compressed (models/cache/kvcomp_encode.py:153-166) -----
+ * The decoder above followed by (sym + min_i) * scale (kvcomp_encode.py:161) in the same kernel: d_out_f16 is
+ * fp16 [tokens, batch, heads, head_dim] = RN16(f32(sym + min_i) * f32(scale)), bit for bit what the two steps
+ * give, without the uint8 tensor in between.  quant_mask / block_size say how (min, scale) are grouped
+ * (any KVC_MASK_* layout). */
+int kvc_decode_dequant(int is_k, const uint8_t *d_encoded, int64_t encoded_bytes,
+                       const uint8_t *d_block_infos, int64_t block_infos_bytes,
+                       const uint8_t *d_thread_infos, int64_t thread_infos_bytes,
+                       const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+                       const int8_t *d_quant_min_ints, const void *d_quant_scales_f16, int quant_mask,
+                       int64_t block_size, void *d_out_f16, int64_t tokens, int64_t batch, int64_t heads,
+                       int64_t head_dim, float *elapsed_ms, void *stream);
+
 /* ---- fused decode + matvec: k_/v_decode_and_mat_vec_mul_cuda_export (kernels.cu:1093-1180) --------
  * K: d_q fp16 [batch, q_heads, head_dim]; d_scores fp16 [batch, q_heads, tokens]:
  *      scores[b,hq,t] = sum_i dequant(K[t,b,hq/rep,i]) * q[b,hq,i]          (kernels.cu:721-776)

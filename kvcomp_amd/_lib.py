@@ -38,6 +38,8 @@ _SIGNATURES = {
                         _u32, _i64p, _i64p, _i64p, _vp],
     "kvc_k_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
+    "kvc_decode_dequant": [_int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _vp, _int, _i64, _vp, _i64, _i64, _i64,
+                           _i64, _f32p, _vp],
     "kvc_k_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,
                                      _i64, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_decode_and_mat_vec_mul": [_vp, _i64, _int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _vp, _int, _vp, _vp,

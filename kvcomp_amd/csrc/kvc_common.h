@@ -55,7 +55,7 @@ constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2
 // ---------------------------------------------------------------------------------------------------
 int kvc_fail(int code, const char *fmt, ...);
 // Tuning knobs settable through kvc_set_option (or, before first use, KVCOMP_<NAME> in the environment).
-enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_COUNT };
+enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_DECODE_PIPELINED = 5, KVC_OPT_COUNT };
 int kvc_option(KvcOption which);
 int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the
@@ -64,6 +64,11 @@ constexpr size_t KVC_WS_SLOT_BYTES = 16384;
 int kvc_workspace_slot(void **slot);
 int kvc_quant_params(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
                      float eb, int8_t *d_min_i8, void *d_scale_f16, void *stream);
+int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+               const uint8_t *d_block_infos, int64_t block_infos_bytes, const uint8_t *d_thread_infos,
+               int64_t thread_infos_bytes, const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_min,
+               const void *d_scale, int quant_mask, void *d_out, int64_t tokens, int64_t batch, int64_t heads,
+               int64_t head_dim, float *elapsed_ms, void *stream);
 int kvc_launch_build_lut(const uint8_t *d_tree, int64_t tree_bytes, int tree_format, uint32_t *d_lut,
                          int n_codebooks, int64_t tree_stride_bytes, hipStream_t stream);
 

@@ -60,6 +60,9 @@ struct KvcFusedArgs {
     int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
     int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
     int double_window;   // refill 64 stream bits at a time where the vector length allows
+    // kvc_expand_kernel (plain decode, decode + dequantize): no x; the operand table holds {scale, min} per element
+    int expand;          // 0: matvec kernels; 1: symbols out (uint8); 2: dequantized values out (fp16)
+    int out_words;       // LDS words per wave for the 32-element output slab
 };
 
 #ifndef KVC_FUSED_OCC1
@@ -337,7 +340,7 @@ struct KvcGeom {
 };
 
 // Issue the global loads of tile (row, col).  bi_off / bi_bn: the tile's block_info words.
-template <int REP, int KIND>
+template <int REP, int KIND, int EXPAND = 0>
 __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
                                                int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw)
 {
@@ -374,12 +377,15 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
         for (int half = 0; half < 2; half++) {
             // per-channel pairs, or one pair per 64-token block (kernels.cu:771-772)
             const int64_t g = a.quant_mask == KVC_MASK_CHANNEL ? tile * D + e0 + half : (int64_t)row;
+            if (EXPAND == 1) continue;                         // symbols out: no quantization parameters
             raw.sc[0][half] = scale16[g];
             raw.mn[0][half] = a.min_i8[g];
         }
+        if (EXPAND == 0) {
 #pragma unroll
-        for (int r = 0; r < REP; r++)
-            raw.x[0][r][0] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
+            for (int r = 0; r < REP; r++)
+                raw.x[0][r][0] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
+        }
     } else {
         const int bh0 = (col * KVC_WAVE) / D;
         const int bh_max = a.batch * a.kv_heads - 1;
@@ -397,11 +403,13 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
                 if (a.quant_mask == KVC_MASK_V_TOKEN) g = tk + half;
                 else if (a.quant_mask == KVC_MASK_SIM_TOKEN) g = (tk + half) * a.batch + b;
                 else g = ((tk + half) * a.batch + b) * a.kv_heads + h;           // KVC_MASK_VECTOR
+                if (EXPAND == 1) continue;
                 raw.sc[s][half] = scale16[g];
                 raw.mn[s][half] = a.min_i8[g];
             }
 #pragma unroll
             for (int r = 0; r < REP; r++) {
+                if (EXPAND != 0) break;
                 const int64_t xrow = (int64_t)b * a.q_heads + h * REP + r;
                 if (KvcGeom<KIND>::SOFTMAX) {
                     const uint2 v = *reinterpret_cast<const uint2 *>(a.scores + xrow * a.scores_stride + tk);
@@ -430,7 +438,7 @@ struct KvcStaged {
 
 // Move a fetched tile into LDS: payload -> packed area (-> per-lane rows), operands -> table; returns the
 // constant terms sum_i min_i * operand_i in bias[].
-template <int REP, int KIND>
+template <int REP, int KIND, int EXPAND = 0>
 __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int row, int col, int lane,
                                                     const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw, float *ops,
                                                     uint32_t *pack, uint32_t *rows, float (&bias)[REP], int &sel_out,
@@ -497,6 +505,16 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
         for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f;
         if (s == 1 && !straddles) continue;                    // no lane of this tile belongs to a second head
         const bool live = KIND != 0 || 2 * lane < D;
+        if (EXPAND == 1) continue;
+        if (EXPAND == 2) {                           // element i of slot s -> {scale, min} at ops[(s * 128 + i) * 2]
+#pragma unroll
+            for (int half = 0; half < 2; half++) {
+                const int i = 2 * lane + half;
+                ops[(s * 128 + i) * 2] = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
+                ops[(s * 128 + i) * 2 + 1] = (float)raw.mn[s][half];
+            }
+            continue;
+        }
         float wgt[REP][2];                           // the two elements' weights: q, p, or exp(score - max)
 #pragma unroll
         for (int r = 0; r < REP; r++) {
@@ -733,6 +751,232 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
 }
 
 // ---------------------------------------------------------------------------------------------------
+// plain decode and decode + dequantize on the same machinery
+//   <- huffman_decode / v_huffman_decode (kvcomp_cuda_extension/src/kernels.cu:602-719), and with DEQ also
+//      the (sym + min) * scale that follows them (models/cache/kvcomp_encode.py:146,161)
+// Tiles are fetched one ahead, staged and decoded exactly as in kvc_fused_kernel; instead of feeding an FMA,
+// every symbol (or its dequantized fp16 value) goes to a 32-element output slab in LDS, which the wave
+// copies out with 8- and 16-byte stores: 32 channels of the tile's 64 tokens (K), or 32 tokens of its 64
+// channels (V).
+// ---------------------------------------------------------------------------------------------------
+// G symbols per half window, 2 G per refill; put(i, g, e) receives the index i of the refill's first element,
+// the element's place g in the refill as a compile-time constant, and the table entry.
+template <int G, bool SKEW, class Put>
+__device__ __forceinline__ void kvc_fast_emit2(const uint32_t *stage, uint32_t &u, uint32_t fentry_base, uint32_t mask4,
+                                               int i0, int n, Put &&put)
+{
+    const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
+    for (int i = i0; i < i0 + n; i += 2 * G) {
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0;
+        kvc_static_for<2 * G>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;
+            if (g == G) R = __builtin_amdgcn_alignbit(hi, lo, es);
+            const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
+            if (g != G - 1 && g != 2 * G - 1) R = __builtin_amdgcn_alignbit(R, R, e);
+            es += e;
+            put(i, g_, e);
+        });
+        u += es & 0xffu;
+    }
+}
+
+// One symbol per refill, table and long-code list in global memory (codes beyond the table index, tiles
+// that do not fit the staging area, windows that may overflow); put1(i, symbol as an fp32 pattern).
+template <bool GSRC, class Put>
+__device__ __forceinline__ void kvc_slow_emit(const uint32_t *words, uint32_t nwords, uint32_t &pos,
+                                           const uint32_t *__restrict__ lut_g, int i0, int n, uint32_t skew, Put &&put1)
+{
+    const uint32_t lshift = 32u - lut_g[0], nlong = lut_g[2];
+    const uint32_t *longs = lut_g + KVC_LUT_HEADER_WORDS;
+    const uint32_t *entries = lut_g + KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS;
+    for (int i = i0; i < i0 + n; i++) {
+        const uint32_t wi = pos >> 5;
+        uint32_t w0 = 0, w1 = 0;
+        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : __brev(words[kvc_skewed(wi, skew)]);
+        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : __brev(words[kvc_skewed(wi + 1, skew)]);
+        const uint32_t hi = (uint32_t)(((((uint64_t)w0) << 32 | w1) << (pos & 31u)) >> 32);
+        const uint32_t e = entries[hi >> lshift];
+        uint32_t len = e & 0xffu, sym = (e >> 8) & 0xffu;
+        if (len == 0) {
+            len = 1;
+            sym = 0;
+            for (uint32_t j = 0; j < nlong; j++) {
+                const uint32_t c = longs[2 * j], ls = longs[2 * j + 1];
+                const uint32_t l = ls & 0xffu;
+                if (((hi ^ c) >> (32u - l)) == 0u) {
+                    len = l;
+                    sym = (ls >> 8) & 0xffu;
+                    break;
+                }
+            }
+        }
+        put1(i, __float_as_uint((float)sym));
+        pos += len;
+    }
+}
+
+// Output slab of one wave, copied to global memory whenever it is full:
+//   K: [64 tokens][SLAB channels], rows one 32-bit word longer than the 64 bytes they carry (so that the lanes'
+//      rows start in all banks); a lane packs the elements of its own row in a register, one word at a time
+//   V: [SLAB tokens][64 channels], dense; consecutive elements of a lane lie a row apart, so they are written singly
+template <bool IS_K, bool DEQ>
+struct KvcSlab {
+    using elem = std::conditional_t<DEQ, uint16_t, uint8_t>;
+    static constexpr int ESZ = (int)sizeof(elem);
+    static constexpr int SLAB = IS_K ? 64 / ESZ : 32;          // elements per lane between two copies
+    static constexpr int K_ROW_WORDS = 64 / 4 + 1;
+    static constexpr int WORDS = IS_K ? 64 * K_ROW_WORDS : SLAB * 64 * ESZ / 4;
+};
+
+template <int KIND, bool DEQ>
+__global__ void __launch_bounds__(KVC_WG, 4) kvc_expand_kernel(KvcFusedArgs a)
+{
+    constexpr bool IS_K = KIND == 0;
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    using S = KvcSlab<IS_K, DEQ>;
+    using elem = typename S::elem;
+    extern __shared__ __align__(16) uint32_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int D = a.head_dim;
+    const int ops_words = DEQ ? SLOTS * 128 * 2 : 0;
+    const int per_wave = ops_words + a.pack_words + KVC_WAVE * a.row_words + a.out_words;
+    uint32_t *s_fentry = smem;
+    float *ops = reinterpret_cast<float *>(smem + a.table_words + wave * per_wave);
+    uint32_t *pack = smem + a.table_words + wave * per_wave + ops_words;
+    uint32_t *rows = pack + a.pack_words;
+    elem *slab = reinterpret_cast<elem *>(rows + KVC_WAVE * a.row_words);
+    const int row = blockIdx.y;
+    const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
+    const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
+    const uint32_t lbits = lut_g[0], nlong = lut_g[2];
+    const bool fast_book = nlong == 0 && lbits <= (uint32_t)KVC_LUT_MAX_BITS && (1u << lbits) <= (uint32_t)a.table_words;
+    if (fast_book)
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) {
+            const uint32_t e = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+            s_fentry[i] = (e & 0xffu) > lbits ? (e & ~0xffu) | lbits : e;
+        }
+    if (lane < KVC_PACK_LEAD) pack[lane] = 0;
+    if (a.row_words) rows[lane * a.row_words] = 0;
+    __syncthreads();
+    const uint32_t mask4 = ((1u << lbits) - 1u) << 2;
+    const int n = IS_K ? D : KVC_V_TOKENS;
+    const uint32_t fe = (uint32_t)(uintptr_t)(kvc_lds_u32 *)s_fentry;
+    const bool fast_loop = fast_book && lut_g[1] <= 7u && n % 8 == 0;     // four codes of <= 7 bits fit a half window
+    const bool wide16 = DEQ || (D & 15) == 0;                 // K rows start on 16-byte boundaries
+    const uint32_t lb = 2u;
+
+    const int T = a.s.tiles_per_wave;
+    const int col0 = (blockIdx.x * KVC_WAVES_PER_WG + wave) * T;
+    int ntiles = a.s.cols - col0;
+    ntiles = ntiles < T ? ntiles : T;
+    if (ntiles <= 0) return;
+    uint32_t bi_off = 0, bi_bn = 0;
+    if (lane < ntiles) {
+        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.s.block_infos + 8 * ((int64_t)row * a.s.cols + col0 + lane));
+        bi_off = bi[0];
+        bi_bn = bi[1];
+    }
+    KvcRaw<1, SLOTS, 1> raw;
+    kvc_fetch_tile<1, KIND, DEQ ? 2 : 1>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    float bias[1];
+    int sel = 0;
+    KvcStaged st = kvc_stage_tile<1, KIND, DEQ ? 2 : 1>(a, row, col0, lane, raw, ops, pack, rows, bias, sel, lb);
+    for (int it = 0; it < ntiles; it++) {
+        const int col = col0 + it;
+        const bool more = it + 1 < ntiles;
+        if (more)
+            kvc_fetch_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
+                                    __builtin_amdgcn_readlane(bi_bn, it + 1), lane, raw);
+        const float *my_ops = ops + sel * 256;
+        const bool fast = fast_loop && st.fits;
+        const uint32_t *words = st.fits ? (a.row_words ? rows + lane * a.row_words : pack) : st.gwords;
+        const uint32_t nw = st.fits ? (uint32_t)(a.row_words ? a.row_words : a.pack_logical) : st.gnwords;
+        const bool skew = st.fits && !a.row_words && a.skew;
+        uint32_t u = st.fits ? st.u0 : st.gpos;                 // fast: lb bits before the code; slow: at the code
+        if (st.fits && !fast) u += lb;
+        // the value of element i: the symbol itself, or (symbol + min_i) * scale_i rounded to fp16
+        auto value = [&](int i, uint32_t e) -> uint32_t {
+            if (DEQ) {
+                const float f = __uint_as_float(e & 0xffffff00u);          // the symbol, exactly
+                const float2 sm = *reinterpret_cast<const float2 *>(my_ops + 2 * i);
+                return (uint32_t)__half_as_ushort(__float2half_rn((f + sm.y) * sm.x));
+            }
+            return (uint32_t)__uint_as_float(e);                           // the low mantissa bits add less than one
+        };
+        uint32_t *slab_w = reinterpret_cast<uint32_t *>(slab);
+        uint32_t cur = 0;
+        // fast loop: element i + g of the lane, g known at compile time
+        auto put = [&](int i, auto g_, uint32_t e) {
+            constexpr int g = decltype(g_)::value;
+            constexpr int PER = 4 / S::ESZ;                                // elements per word
+            const uint32_t v = value(i + g, e);
+            if (IS_K) {
+                cur = (g % PER == 0) ? v : cur | (v << (8 * S::ESZ * (g % PER)));
+                if (g % PER == PER - 1)
+                    slab_w[lane * S::K_ROW_WORDS + ((i & (S::SLAB - 1)) + g) / PER] = cur;
+            } else {
+                slab[((i + g) & (S::SLAB - 1)) * KVC_WAVE + lane] = (elem)v;
+            }
+        };
+        // slow loop: one element at a time
+        auto put1 = [&](int i, uint32_t e) {
+            const int j = i & (S::SLAB - 1);
+            slab[IS_K ? lane * (S::K_ROW_WORDS * 4 / S::ESZ) + j : j * KVC_WAVE + lane] = (elem)value(i, e);
+        };
+        for (int i0 = 0; i0 < n; i0 += S::SLAB) {
+            const int len = n - i0 < S::SLAB ? n - i0 : S::SLAB;
+            if (fast) {
+                if (skew) kvc_fast_emit2<4, true>(words, u, fe, mask4, i0, len, put);
+                else kvc_fast_emit2<4, false>(words, u, fe, mask4, i0, len, put);
+            } else if (st.fits) {
+                kvc_slow_emit<false>(words, nw, u, lut_g, i0, len, skew ? (uint32_t)a.skew : 0u, put1);
+            } else {
+                kvc_slow_emit<true>(words, nw, u, lut_g, i0, len, 0u, put1);
+            }
+            kvc_wave_sync();
+            // ---- copy the slab out, 16 bytes per lane and store
+            constexpr int PER16 = 16 / S::ESZ;                             // elements per piece
+            if (IS_K) {
+                // rows of `len` elements (64 bytes when full): four lanes per row
+                elem *out = reinterpret_cast<elem *>(a.out) + (int64_t)row * KVC_WAVE * a.s.stride + (int64_t)col * D + i0;
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int f = lane + KVC_WAVE * t, r = f >> 2, c = f & 3;
+                    if (c * PER16 < len) {
+                        const uint32_t *src = slab_w + r * S::K_ROW_WORDS + 4 * c;
+                        uint4 v = make_uint4(src[0], src[1], src[2], src[3]);
+                        elem *dst = out + (int64_t)r * a.s.stride + c * PER16;
+                        if (wide16) {
+                            *reinterpret_cast<uint4 *>(dst) = v;
+                        } else {                                            // uint8 rows with head_dim % 16 == 8: 8-byte alignment only
+                            *reinterpret_cast<uint2 *>(dst) = make_uint2(v.x, v.y);
+                            if (c * PER16 + PER16 <= len) *reinterpret_cast<uint2 *>(dst + 8) = make_uint2(v.z, v.w);
+                        }
+                    }
+                }
+            } else {
+                constexpr int PIECES = KVC_WAVE / PER16;                    // pieces per row of 64 channels
+                elem *out = reinterpret_cast<elem *>(a.out) + ((int64_t)row * KVC_V_TOKENS + i0) * a.s.stride + (int64_t)col * KVC_WAVE;
+#pragma unroll
+                for (int t = 0; t < S::SLAB * PIECES / KVC_WAVE; t++) {
+                    const int f = lane + KVC_WAVE * t, r = f / PIECES, c = f - r * PIECES;
+                    if (r < len) {
+                        const uint4 v = *reinterpret_cast<const uint4 *>(slab + r * KVC_WAVE + c * PER16);
+                        *reinterpret_cast<uint4 *>(out + (int64_t)r * a.s.stride + c * PER16) = v;
+                    }
+                }
+            }
+            kvc_wave_sync();
+        }
+        if (more) st = kvc_stage_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel, lb);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------------------------
 template <int REP>
@@ -750,7 +994,7 @@ static void kvc_launch_fused(int kind, const KvcFusedArgs &a, dim3 grid, size_t 
 // longest lane stream); without them from twice the payload's means.  Tiles that do not fit are decoded
 // from global memory, so the sizes only affect speed.  Everything stays within 64 KiB per workgroup.
 static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_bytes, int64_t tiles,
-                           int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits)
+                           int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t extra_words = 0)
 {
     const int force_rows = kvc_option(KVC_OPT_FUSED_ROWS);   // 0 / 1 overrides the choice below
     a.table_words = 1 << ((max_code_bits >= 1 && max_code_bits <= KVC_LUT_MAX_BITS) ? max_code_bits : KVC_LUT_MAX_BITS);
@@ -758,15 +1002,18 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     // room for the two-symbol table (8 bytes per index of 2 * longest-code bits) when the codes are short
     const int pair_limit = kvc_option(KVC_OPT_FUSED_PAIR_BITS);
     a.pair_bits = 0;
+    a.expand = 0;
+    a.out_words = 0;
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
-    if (max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
+    if (extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
         a.pair_bits = 2 * max_code_bits;
         if (a.table_words < (2 << a.pair_bits)) a.table_words = 2 << a.pair_bits;
     }
-    const int64_t ops_words = (int64_t)slots * 128 * rep;
+    const int64_t ops_words = (int64_t)slots * 128 * rep + extra_words;   // per wave, besides the payload
     const int64_t budget = (65536 / 4 - a.table_words - KVC_LDS_SLACK_WORDS) / KVC_WAVES_PER_WG - ops_words;   // words per wave
     const int64_t mean_tile = encoded_bytes / (tiles > 0 ? tiles : 1);
-    int64_t tile_bytes = max_tile_bytes > 0 ? max_tile_bytes : 2 * mean_tile + 64;
+    // without the encoder's figure: tiles hold thousands of symbols, so their sizes stay close to the mean
+    int64_t tile_bytes = max_tile_bytes > 0 ? max_tile_bytes : mean_tile + mean_tile / 4 + 256;
     if (tile_bytes > KVC_MAX_TILE_BYTES) tile_bytes = KVC_MAX_TILE_BYTES;
     // lead words + the payload's chunks (it may start anywhere in its first chunk) + look-ahead
     int64_t pack = KVC_PACK_LEAD + ((tile_bytes + 15 + 15) / 16) * 4 + 4;   // three look-ahead words, rounded up
@@ -892,6 +1139,71 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
         case 4: kvc_launch_fused<4>(kind, a, grid, lds, stream); break;
         default: kvc_launch_fused<8>(kind, a, grid, lds, stream); break;
     }
+    KVC_HIP(hipGetLastError());
+    return timer.finish();
+}
+
+// Plain decode (d_out uint8 [tokens, stride]) or decode + dequantize (d_out fp16, same shape) of a whole stream.
+// Returns 1 when the layout is not one the kernel handles (the caller then uses the two-step kernels).
+int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,
+               const uint8_t *d_block_infos, int64_t block_infos_bytes, const uint8_t *d_thread_infos,
+               int64_t thread_infos_bytes, const uint8_t *d_encoded, int64_t encoded_bytes, const int8_t *d_min,
+               const void *d_scale, int quant_mask, void *d_out, int64_t tokens, int64_t batch, int64_t heads,
+               int64_t head_dim, float *elapsed_ms, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    if (head_dim <= 0 || head_dim > KVC_K_VEC_LEN || head_dim % 8 != 0) return 1;
+    if (deq) {
+        if (is_k && quant_mask != KVC_MASK_K_BLOCK && quant_mask != KVC_MASK_CHANNEL) return 1;
+        if (!is_k && quant_mask != KVC_MASK_V_TOKEN && quant_mask != KVC_MASK_SIM_TOKEN && quant_mask != KVC_MASK_VECTOR) return 1;
+    }
+    void *slot = nullptr;
+    if (int rc = kvc_workspace_slot(&slot)) return rc;
+    KvcFusedArgs a;
+    int64_t rows;
+    const int64_t stride = batch * heads * head_dim;
+    if (int rc = kvc_fill_stream_args(a.s, d_encoded, encoded_bytes, d_block_infos, block_infos_bytes, d_thread_infos,
+                                      thread_infos_bytes, (const uint32_t *)slot, is_k, tokens, stride, head_dim, &rows))
+        return rc;
+    KVC_REQUIRE(((uintptr_t)d_out & 15) == 0, "output pointer must be 16-byte aligned");
+    a.min_i8 = d_min;
+    a.scale = reinterpret_cast<const __half *>(d_scale);
+    a.quant_mask = deq ? quant_mask : (is_k ? KVC_MASK_K_BLOCK : KVC_MASK_V_TOKEN);
+    a.x = nullptr;
+    a.out = d_out;
+    a.out_f32 = 0;
+    a.out_stride = 0;
+    a.scores = nullptr;
+    a.scores_stride = 0;
+    a.sm_scale = 1.f;
+    a.ml = nullptr;
+    a.tokens = tokens;
+    a.batch = (int)batch;
+    a.kv_heads = (int)heads;
+    a.q_heads = (int)heads;
+    a.head_dim = (int)head_dim;
+    const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
+    const int out_words = is_k ? (deq ? KvcSlab<true, true>::WORDS : KvcSlab<true, false>::WORDS)
+                               : (deq ? KvcSlab<false, true>::WORDS : KvcSlab<false, false>::WORDS);
+    const size_t lds = kvc_plan_lds(a, slots, deq ? 2 : 0, encoded_bytes, rows * a.s.cols, 0, 0, 0, out_words);
+    a.expand = deq ? 2 : 1;
+    a.out_words = out_words;
+    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
+    KvcTimer timer(elapsed_ms, stream);
+    if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
+    const dim3 grid = kvc_grid(a.s, rows);
+    const int kind = is_k ? 0 : slots;
+#define KVC_EXPAND_LAUNCH(K, Q) hipLaunchKernelGGL((kvc_expand_kernel<K, Q>), grid, dim3(KVC_WG), lds, stream, a)
+    if (deq) {
+        if (kind == 0) KVC_EXPAND_LAUNCH(0, true);
+        else if (kind == 1) KVC_EXPAND_LAUNCH(1, true);
+        else KVC_EXPAND_LAUNCH(2, true);
+    } else {
+        if (kind == 0) KVC_EXPAND_LAUNCH(0, false);
+        else if (kind == 1) KVC_EXPAND_LAUNCH(1, false);
+        else KVC_EXPAND_LAUNCH(2, false);
+    }
+#undef KVC_EXPAND_LAUNCH
     KVC_HIP(hipGetLastError());
     return timer.finish();
 }

@@ -50,6 +50,7 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"fused_pair_bits", "KVCOMP_FUSED_PAIR_BITS", 8},            // widest two-symbol table index; 0 = one symbol per look-up
     {"fused_double_window", "KVCOMP_FUSED_DOUBLE_WINDOW", 1},    // 64 stream bits per refill in the one-symbol loops
     {"fused_skew", "KVCOMP_FUSED_SKEW", -1},                     // skewed payload layout: -1 choose per call, 0 never, 1 always
+    {"decode_pipelined", "KVCOMP_DECODE_PIPELINED", 1},          // plain decode / decode + dequantize on the fused kernels' machinery
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;

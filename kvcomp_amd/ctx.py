@@ -326,8 +326,19 @@ class KVCompCtx:
                   self.head_num, self.head_dim)
         return decoded, t_ms
 
+    # decode and dequantize in one kernel (no uint8 tensor in between); False = the reference's two steps
+    fused_get = True
+
     def get_only_compressed(self) -> Tuple[torch.Tensor, float]:
         """kvcomp_encode.py:153-166: decode + dequantize the compressed part -> ([ctx_c, B, H, D] fp16, ms)."""
+        if KVCompCtx.fused_get:
+            self._assert_ready()
+            out = torch.empty(self.compressed_ctx_len, self.batch_size, self.head_num, self.head_dim, dtype=torch.float16,
+                              device=self.device)
+            t_ms = kvcomp_cuda.decode_dequant(self.is_k, self.encoded_data, self.block_infos, self.thread_infos,
+                                              self.decode_codebook, self.quant_min_ints, self.quant_scales,
+                                              dims_to_mask(self.quant_dims), self.block_size, out)
+            return out, t_ms
         decoded, t_ms = self.get_decode_quant_ints()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()

@@ -213,6 +213,27 @@ def v_entropy_decode_cuda_export(in_tensor, block_infos, thread_infos, decode_co
     return _entropy_decode(False, in_tensor, block_infos, thread_infos, decode_code_book, out, head_num, head_dim, tree_format)
 
 
+def decode_dequant(is_k: bool, in_tensor, block_infos, thread_infos, decode_code_book, quant_min_ints, quant_scales,
+                   quant_mask: int, block_size: int, out: torch.Tensor, tree_format: int = TREE_I8) -> float:
+    """Huffman decode + (sym + min) * scale in one kernel (models/cache/kvcomp_encode.py:153-166 without the
+    uint8 tensor in between).  out: device fp16 [T, B, H, D]; returns elapsed milliseconds."""
+    for t, n in ((in_tensor, "in_tensor"), (block_infos, "block_infos"), (thread_infos, "thread_infos"),
+                 (decode_code_book, "decode_code_book")):
+        _dev_u8(t, n)
+    _require(out.is_cuda and out.dtype == torch.float16 and out.dim() == 4 and out.is_contiguous(),
+             "out must be a contiguous device float16 tensor [T, B, H, D]")
+    _require(quant_min_ints.dtype == torch.int8 and quant_scales.dtype == torch.float16, "min_ints int8, scales fp16")
+    T, B, H, D = out.shape
+    ms = C.c_float(0.0)
+    with torch.cuda.device(out.device):
+        check(_lib.lib().kvc_decode_dequant(int(is_k), _ptr(in_tensor), in_tensor.numel(), _ptr(block_infos), block_infos.numel(),
+                                            _ptr(thread_infos), thread_infos.numel(), _ptr(decode_code_book),
+                                            decode_code_book.numel(), tree_format, _ptr(quant_min_ints.contiguous()),
+                                            _ptr(quant_scales.contiguous()), quant_mask, block_size, _ptr(out), T, B, H, D,
+                                            C.byref(ms), _stream(out)))
+    return ms.value
+
+
 def _fused(is_k, decode_code_book, block_infos, thread_infos, encoded_data, quant_min_ints, quant_scales, B, Cout,
            head_num, head_dim, tree_format):
     for t, n in ((decode_code_book, "decode_code_book"), (block_infos, "block_infos"), (thread_infos, "thread_infos"),

@@ -277,3 +277,29 @@ def test_one_call_attention_grows_with_the_cache():
             s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
             ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
             assert (out - ref).abs().max() <= 3e-3 * ref.abs().max(), "step %d" % i
+
+
+@pytest.mark.parametrize("is_k,mode,B,H,D", [(True, "ChannelQuant", 2, 3, 96), (True, "BlockQuant", 1, 4, 128),
+                                              (False, "TokenQuant", 2, 3, 96), (False, "VectorQuant", 2, 4, 128)])
+def test_one_kernel_get_equals_decode_then_dequant(is_k, mode, B, H, D):
+    """kvc_decode_dequant against the reference's two steps (kvcomp_encode.py:153-166) and against the oracle."""
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode=mode if is_k else "BlockQuant", v_mode=mode if not is_k else "TokenQuant")
+    T = 512
+    x = (S.synth_k if is_k else S.synth_v)(T, B, H, D)
+    ctx = KVCompCtx(is_k, B, H, D, 0.1)
+    ctx.store(x.to(DEV))
+    assert ctx.compressed_ctx_len == T
+    try:
+        KVCompCtx.fused_get = True
+        one, _ = ctx.get_only_compressed()
+        KVCompCtx.fused_get = False
+        two, _ = ctx.get_only_compressed()
+    finally:
+        KVCompCtx.fused_get = True
+    assert one.shape == two.shape == (T, B, H, D)
+    assert torch.equal(one.view(torch.int16), two.view(torch.int16))
+    mask = _oracle_mask(ctx)
+    o = O.quant(S.np16(S.blocked(x, ctx.block_size)), mask, 0.1)
+    deq = O.dequant(o[3], o[4], o[2], mask).reshape(T, B, H, D)
+    assert np.array_equal(one.cpu().numpy().view(np.uint16), deq.view(np.uint16))
