@@ -60,10 +60,22 @@ const char *kvc_last_error(void);
 int kvc_abi_version(void);
 /* Tuning knobs (no counterpart in the reference).  Each can also be preset through the environment
  * variable KVCOMP_<NAME IN CAPITALS>, read once on first use.
- *   "fused_rows":           -1 (default) the fused decoders decide per call whether to re-lay a tile's lane
- *                           streams as LDS rows; 0 never; 1 whenever the rows fit.
- *   "fused_tiles_per_wave":  0 (default) chosen per call; n > 0: consecutive tiles one wave works through. */
+ *   "fused_rows":           1: the fused decoders re-lay a tile's lane streams as LDS rows an odd number of words
+ *                           apart whenever they fit; otherwise (default -1) never.
+ *   "fused_skew":           -1 (default) decided per call: the tile payload is staged with two spare words after
+ *                           every 32 when the mean stream length would otherwise line the lanes up on a few LDS
+ *                           banks; 0 never; 1 always.
+ *   "fused_tiles_per_wave":  0 (default) chosen per call; n > 0: consecutive tiles one wave works through.
+ *   "fused_pair_bits":       widest index of the two-symbols-per-look-up table (default 8; 0 = one symbol per look-up).
+ *   "fused_double_window":   1 (default): 64 stream bits per refill in the one-symbol loops; 0: 32.
+ *   "fused_rounded":         0 (default): the fused matvecs multiply q / p by (sym + min) * scale as it stands, in
+ *                           fp32.  1: every such value is first rounded to fp16, as the reference's dequantizer
+ *                           rounds it (models/cache/kvcomp_encode.py:146), so the result is the fp32 attention
+ *                           over that fp16 cache; about half the speed.
+ *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile
+ *                           pipeline; 0: on the simpler stand-alone kernels. */
 int kvc_set_option(const char *name, int value);
+int kvc_get_option(const char *name, int *value);
 
 /* ---- sizes: calculate_buffer_size (kernels.cu:893-917) --------------------------------------------
  * out4 = {block_infos bytes, thread_infos bytes, idx_offset bytes (8), payload pre-allocation bytes}. */

@@ -28,6 +28,7 @@ class CompressedDesc(C.Structure):
 _SIGNATURES = {
     "kvc_abi_version": [],
     "kvc_set_option": [C.c_char_p, _int],
+    "kvc_get_option": [C.c_char_p, _intp],
     "kvc_calculate_buffer_size": [_i64, _i64, _int, _i64, _i64, _i64p],
     "kvc_histogram": [_vp, _i64, _vp, _vp],
     "kvc_build_codebook_host": [_i64p, _int, _intp, _vp, _i64, _i64p, _vp, _i64, _i64p],
@@ -89,6 +90,14 @@ def lib():
             fn.restype = _RESTYPES.get(name, _int)
         _LIB = L
     return _LIB
+
+
+def set_option(name: str, value: int) -> int:
+    """Set a tuning knob of the library (see include/kvcomp_hip.h); returns the previous value."""
+    old = C.c_int(0)
+    check(lib().kvc_get_option(name.encode(), C.byref(old)))
+    check(lib().kvc_set_option(name.encode(), int(value)))
+    return old.value
 
 
 def check(rc):

@@ -61,6 +61,10 @@ struct KvcFusedArgs {
     int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
     int double_window;   // refill 64 stream bits at a time where the vector length allows
     // kvc_expand_kernel (plain decode, decode + dequantize): no x; the operand table holds {scale, min} per element
+    // Rounded mode of the matvec kernels: every (sym + min) * scale is rounded to fp16 before it meets q / p, as the
+    // reference's dequantizer does (models/cache/kvcomp_encode.py:146); the operand table then holds
+    // {min, scale, weight of each query head} per element and nothing is folded into a constant term.
+    int rounded;
     int expand;          // 0: matvec kernels; 1: symbols out (uint8); 2: dequantized values out (fp16)
     int out_words;       // LDS words per wave for the 32-element output slab
 };
@@ -130,7 +134,7 @@ struct KvcVec {
 template <int REP, bool GSRC>
 __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_t nwords, uint32_t pos,
                                                   const uint32_t *__restrict__ lut_g, int n, const float *ops,
-                                                  uint32_t skew)
+                                                  uint32_t skew, bool rounded)
 {
     const uint32_t lshift = 32u - lut_g[0], nlong = lut_g[2];
     const uint32_t *longs = lut_g + KVC_LUT_HEADER_WORDS;
@@ -161,8 +165,15 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
             }
         }
         const float f = (float)sym;
+        if (rounded) {
+            const float *o = ops + i * (REP + 2);
+            const float v = __half2float(__float2half_rn((f + o[0]) * o[1]));
 #pragma unroll
-        for (int r = 0; r < REP; r++) acc.v[r] = fmaf(f, ops[i * REP + r], acc.v[r]);
+            for (int r = 0; r < REP; r++) acc.v[r] = fmaf(v, o[2 + r], acc.v[r]);
+        } else {
+#pragma unroll
+            for (int r = 0; r < REP; r++) acc.v[r] = fmaf(f, ops[i * REP + r], acc.v[r]);
+        }
         pos += len;
     }
     return acc;
@@ -281,6 +292,35 @@ __device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t &u
             worst = m > worst ? m : worst;
         }
         u += used;
+    }
+}
+
+// Rounded mode: the dequantized value is rounded to fp16 before the multiplication (see KvcFusedArgs::rounded).
+// Four symbols per refill (codes of at most 7 bits); the element's {min, scale, weights} come from one address
+// for the whole wave.
+template <bool SKEW, int REP>
+__device__ __forceinline__ void kvc_rounded_dot(const uint32_t *stage, uint32_t &u, uint32_t fentry_base, uint32_t mask4,
+                                                int n, const float *ops, float (&acc)[REP])
+{
+    constexpr int OPS = REP + 2;
+    const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
+    for (int i = 0; i < n; i += 4) {
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1];
+        uint32_t R = __builtin_amdgcn_alignbit(w1, w0, u);
+        uint32_t es = 0;
+        kvc_static_for<4>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;
+            const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
+            R = __builtin_amdgcn_alignbit(R, R, e);
+            es += e;
+            const float f = __uint_as_float(e & 0xffffff00u);              // the symbol, exactly
+            const float *o = ops + (i + g) * OPS;
+            const float v = __half2float(__float2half_rn((f + o[0]) * o[1]));
+#pragma unroll
+            for (int r = 0; r < REP; r++) acc[r] = fmaf(v, o[2 + r], acc[r]);
+        });
+        u += es & 0xffu;
     }
 }
 
@@ -544,6 +584,14 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
             const int i = 2 * lane + half;
             const float sc = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
             const float mn = (float)raw.mn[s][half];
+            if (a.rounded) {                             // wave-uniform
+                float *o = ops + (s * 128 + i) * (REP + 2);
+                o[0] = mn;
+                o[1] = sc;
+#pragma unroll
+                for (int r = 0; r < REP; r++) o[2 + r] = wgt[r][half];
+                continue;
+            }
 #pragma unroll
             for (int r = 0; r < REP; r++) {
                 const float v = sc * wgt[r][half];
@@ -601,10 +649,11 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int D = a.head_dim;
-    const int per_wave = SLOTS * 128 * REP + a.pack_words + KVC_WAVE * a.row_words;
+    const int ops_per_elem = a.rounded ? REP + 2 : REP;
+    const int per_wave = SLOTS * 128 * ops_per_elem + a.pack_words + KVC_WAVE * a.row_words;
     uint32_t *s_fentry = smem;
     float *ops = reinterpret_cast<float *>(smem + a.table_words + wave * per_wave);
-    uint32_t *pack = smem + a.table_words + wave * per_wave + SLOTS * 128 * REP;
+    uint32_t *pack = smem + a.table_words + wave * per_wave + SLOTS * 128 * ops_per_elem;
     uint32_t *rows = pack + a.pack_words;
     const int row = blockIdx.y;
     const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
@@ -620,7 +669,7 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
     };
     // two symbols per look-up when every pair of codes fits the pair table's index
     const uint32_t pbits = 2u * lut_g[1];
-    const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && lbits <= 7u;
+    const bool pairs = fast_book && !a.rounded && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && lbits <= 7u;
     if (pairs) {
         // the single-symbol table goes to the (not yet used) per-wave areas, the pair table is derived from it
         uint32_t *tmp = smem + a.table_words;
@@ -671,12 +720,17 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
         if (more)   // loads for the next tile fly while this one is decoded
             kvc_fetch_tile<REP, KIND>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
                                       __builtin_amdgcn_readlane(bi_bn, it + 1), lane, raw);
-        const float *my_ops = ops + sel * 128 * REP;
+        const float *my_ops = ops + sel * 128 * ops_per_elem;
         float acc[REP];
 #pragma unroll
         for (int r = 0; r < REP; r++) acc[r] = 0.f;
-        bool redo = !(fast_book && st.fits);
-        if (!redo) {
+        bool redo = !(fast_book && st.fits) || (a.rounded && lut_g[1] > 7u);
+        if (!redo && a.rounded) {
+            const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
+            uint32_t u = st.u0;
+            if (!a.row_words && a.skew) kvc_rounded_dot<true, REP>(words, u, fe, mask4, n, my_ops, acc);
+            else kvc_rounded_dot<false, REP>(words, u, fe, mask4, n, my_ops, acc);
+        } else if (!redo) {
             const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
             const bool skew = !a.row_words && a.skew;
             uint32_t u = st.u0, worst = 0;
@@ -711,9 +765,9 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
             if (st.fits) {
                 const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
                 const uint32_t nw = (uint32_t)(a.row_words ? a.row_words : a.pack_logical);
-                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + lb, lut_g, n, my_ops, a.row_words ? 0u : (uint32_t)a.skew);
+                res = kvc_slow_tile<REP, false>(words, nw, st.u0 + lb, lut_g, n, my_ops, a.row_words ? 0u : (uint32_t)a.skew, a.rounded != 0);
             } else {
-                res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops, 0u);
+                res = kvc_slow_tile<REP, true>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_ops, 0u, a.rounded != 0);
             }
 #pragma unroll
             for (int r = 0; r < REP; r++) acc[r] = res.v[r];
@@ -1002,6 +1056,7 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     // room for the two-symbol table (8 bytes per index of 2 * longest-code bits) when the codes are short
     const int pair_limit = kvc_option(KVC_OPT_FUSED_PAIR_BITS);
     a.pair_bits = 0;
+    a.rounded = 0;
     a.expand = 0;
     a.out_words = 0;
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
@@ -1125,8 +1180,10 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     a.head_dim = (int)head_dim;
     const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
     const int kind = is_k ? 0 : (a.scores ? 2 : 0) + slots;
-    const size_t lds = kvc_plan_lds(a, slots, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
-                                    max_stream_bytes, max_code_bits);
+    const int rounded = kvc_option(KVC_OPT_FUSED_ROUNDED) != 0;
+    const size_t lds = kvc_plan_lds(a, slots, rounded ? (int)rep + 2 : (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
+                                    max_stream_bytes, rounded ? 0 : max_code_bits);
+    a.rounded = rounded;
     a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
     KvcTimer timer(elapsed_ms, stream);
     if (!d_luts) {

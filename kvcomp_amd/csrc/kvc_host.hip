@@ -51,6 +51,7 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"fused_double_window", "KVCOMP_FUSED_DOUBLE_WINDOW", 1},    // 64 stream bits per refill in the one-symbol loops
     {"fused_skew", "KVCOMP_FUSED_SKEW", -1},                     // skewed payload layout: -1 choose per call, 0 never, 1 always
     {"decode_pipelined", "KVCOMP_DECODE_PIPELINED", 1},          // plain decode / decode + dequantize on the fused kernels' machinery
+    {"fused_rounded", "KVCOMP_FUSED_ROUNDED", 0},                // 1: round each dequantized value to fp16 before the matvec (slower)
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;
@@ -76,6 +77,19 @@ extern "C" int kvc_set_option(const char *name, int value)
     for (int i = 0; i < KVC_OPT_COUNT; i++) {
         if (std::strcmp(name, g_option_defs[i].name) == 0) {
             g_options[i].store(value);
+            return 0;
+        }
+    }
+    return kvc_fail(-1, "unknown option '%s'", name);
+}
+
+extern "C" int kvc_get_option(const char *name, int *value)
+{
+    KVC_REQUIRE(name != nullptr && value != nullptr, "NULL argument");
+    std::call_once(g_options_once, init_options);
+    for (int i = 0; i < KVC_OPT_COUNT; i++) {
+        if (std::strcmp(name, g_option_defs[i].name) == 0) {
+            *value = g_options[i].load();
             return 0;
         }
     }
