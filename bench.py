@@ -334,6 +334,23 @@ def main():
     log("[bench] step %.3f ms; fused K kernel %.3f ms (%.1f GB/s compressed), fused V kernel %.3f ms (%.1f GB/s compressed)"
         % (ms_per_step, k_ms, kb / k_ms / 1e6, v_ms, vb / v_ms / 1e6))
     assert torch.isfinite(out).all()
+    # the same pass in rounded mode: every dequantized value is rounded to fp16 before it meets q / p, as the
+    # reference's dequantizer rounds it (models/cache/kvcomp_encode.py:146)
+    from kvcomp_amd import _lib
+    was = _lib.set_option("fused_rounded", 1)
+    try:
+        attn_r = A.CompressedAttention(kctx, vctx)
+        for _ in range(args.warmup):
+            attn_r.attend(q)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            attn_r.attend(q)
+        torch.cuda.synchronize()
+        rounded_ms = (time.perf_counter() - t0) / args.steps * 1e3
+    finally:
+        _lib.set_option("fused_rounded", was)
+    log("[bench] rounded mode: step %.3f ms" % rounded_ms)
 
     # template arguments: query heads per KV head, then 0 = K tile, 3 / 4 = V tile with the softmax on the fly
     # (4: head_dim is not a multiple of 64, tiles may straddle two heads)
@@ -354,6 +371,11 @@ def main():
                                         "fp16_equivalent_GBs": round(4 * numel / (ms_per_step * 1e-3) / 1e9, 1),
                                         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
                                         "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)},
+                                        "arithmetic": "q . ((sym + min) * scale) with the dequantized value kept in fp32 (within 1e-4 of "
+                                                      "fp64 attention over that dequantization); rounded_mode rounds it to fp16 first like "
+                                                      "the reference's dequantizer (within 1e-3 of fp32 attention over the fp16 cache)",
+                                        "rounded_mode": {"ms_per_step": round(rounded_ms, 4),
+                                                         "GBs": round((kb + vb) / (rounded_ms * 1e-3) / 1e9, 1)},
                                         "symbols_per_s": {"fused_k": round(numel / k_ms * 1e3), "fused_v": round(numel / v_ms * 1e3)},
                                         "codec": rates},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
