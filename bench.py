@@ -173,9 +173,9 @@ def codec_rates(kctx, vctx, k, v, cfg):
 # what the same counter reads for the 256 MiB kvc_calibration_copy_kernel of the same run (FETCH_SIZE x2.0,
 # WRITE_SIZE x1.0).  Source: profiles/fused_decode_attention_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2": {"kvc_fused_kernel<1, 0>": int((4041.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2696.9 * 2.0 + 528.0) * 1024)},
-    "cfg3": {"kvc_fused_kernel<4, 0>": int((31585.3 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, 3>": int((26270.6 * 2.0 + 16800.3) * 1024)},
-    "cfg5": {"kvc_fused_kernel<1, 0>": int((102429.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((46666.7 * 2.0 + 12778.7) * 1024)},
+    "cfg2": {"kvc_fused_kernel<1, 0>": int((4074.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2733.4 * 2.0 + 528.0) * 1024)},
+    "cfg3": {"kvc_fused_kernel<4, 0>": int((31646.6 * 2.0 + 18432.0) * 1024), "kvc_fused_kernel<4, 3>": int((27569.6 * 2.0 + 27055.6) * 1024)},
+    "cfg5": {"kvc_fused_kernel<1, 0>": int((102470.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((45729.2 * 2.0 + 18279.0) * 1024)},
 }
 
 
@@ -258,6 +258,8 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eb-k", type=float, default=None, help="override the K error bound of the workload (cfg5 sweeps 0.05 / 0.1 / 0.2)")
+    ap.add_argument("--no-rounded", action="store_true",
+                    help="skip the extra pass in rounded mode (keeps a kernel trace of this run to one variant per kernel)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 256 MiB device copy (kvc_calibration_copy_kernel), the yardstick "
                          "for FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -337,20 +339,22 @@ def main():
     # the same pass in rounded mode: every dequantized value is rounded to fp16 before it meets q / p, as the
     # reference's dequantizer rounds it (models/cache/kvcomp_encode.py:146)
     from kvcomp_amd import _lib
-    was = _lib.set_option("fused_rounded", 1)
-    try:
-        attn_r = A.CompressedAttention(kctx, vctx)
-        for _ in range(args.warmup):
-            attn_r.attend(q)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            attn_r.attend(q)
-        torch.cuda.synchronize()
-        rounded_ms = (time.perf_counter() - t0) / args.steps * 1e3
-    finally:
-        _lib.set_option("fused_rounded", was)
-    log("[bench] rounded mode: step %.3f ms" % rounded_ms)
+    rounded_ms = None
+    if not args.no_rounded:
+        was = _lib.set_option("fused_rounded", 1)
+        try:
+            attn_r = A.CompressedAttention(kctx, vctx)
+            for _ in range(args.warmup):
+                attn_r.attend(q)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                attn_r.attend(q)
+            torch.cuda.synchronize()
+            rounded_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        finally:
+            _lib.set_option("fused_rounded", was)
+        log("[bench] rounded mode: step %.3f ms" % rounded_ms)
 
     # template arguments: query heads per KV head, then 0 = K tile, 3 / 4 = V tile with the softmax on the fly
     # (4: head_dim is not a multiple of 64, tiles may straddle two heads)
@@ -374,8 +378,8 @@ def main():
                                         "arithmetic": "q . ((sym + min) * scale) with the dequantized value kept in fp32 (within 1e-4 of "
                                                       "fp64 attention over that dequantization); rounded_mode rounds it to fp16 first like "
                                                       "the reference's dequantizer (within 1e-3 of fp32 attention over the fp16 cache)",
-                                        "rounded_mode": {"ms_per_step": round(rounded_ms, 4),
-                                                         "GBs": round((kb + vb) / (rounded_ms * 1e-3) / 1e9, 1)},
+                                        "rounded_mode": None if rounded_ms is None else
+                                        {"ms_per_step": round(rounded_ms, 4), "GBs": round((kb + vb) / (rounded_ms * 1e-3) / 1e9, 1)},
                                         "symbols_per_s": {"fused_k": round(numel / k_ms * 1e3), "fused_v": round(numel / v_ms * 1e3)},
                                         "codec": rates},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
