@@ -69,8 +69,17 @@ struct KvcFusedArgs {
     int out_words;       // LDS words per wave for the 32-element output slab
 };
 
-#ifndef KVC_FUSED_OCC1
-#define KVC_FUSED_OCC1 5   // workgroups per CU the REP = 1 kernels are compiled for (6 spills)
+// Workgroups per CU (= waves per SIMD) each matvec kernel is compiled for.  With one query head per KV head the
+// decode loops wait on LDS round trips and every further wave pays, so those kernels get the most their register
+// demand allows without spilling (kinds 2 - 4 carry a second operand table or the softmax).  With four query heads
+// the four FMAs per symbol hide the round trip; measured, 4 and 5 waves tie and 6 or 7 are 6 - 8 % slower.
+constexpr int kvc_fused_occupancy(int rep, int kind)
+{
+    const bool two_slots = kind == 2 || kind == 4;
+    return rep == 1 ? (kind == 1 ? 8 : 7) : (rep == 2 || (rep == 4 && !two_slots)) ? 5 : 1;
+}
+#ifndef KVC_FUSED_OCC
+#define KVC_FUSED_OCC(REP, KIND) kvc_fused_occupancy(REP, KIND)
 #endif
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
@@ -639,7 +648,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 }
 
 template <int REP, int KIND>
-__global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 || (REP == 4 && KvcGeom<KIND>::SLOTS == 1)) ? 5 : 1) kvc_fused_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
@@ -717,9 +726,14 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
     for (int it = 0; it < ntiles; it++) {
         const int col = col0 + it;
         const bool more = it + 1 < ntiles;
+        // The lane number is made opaque per tile: otherwise every address the fetch and the staging derive from
+        // it is hoisted out of this loop and held in a register of its own through the decode loops (some twenty
+        // registers, i.e. two waves per SIMD less)
+        int lane_f = lane;
+        asm volatile("" : "+v"(lane_f));
         if (more)   // loads for the next tile fly while this one is decoded
             kvc_fetch_tile<REP, KIND>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
-                                      __builtin_amdgcn_readlane(bi_bn, it + 1), lane, raw);
+                                      __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
         const float *my_ops = ops + sel * 128 * ops_per_elem;
         float acc[REP];
 #pragma unroll
@@ -799,7 +813,9 @@ __global__ void __launch_bounds__(KVC_WG, REP == 1 ? KVC_FUSED_OCC1 : (REP <= 2 
         }
         if (more) {
             kvc_wave_sync();     // every lane is done reading this tile's LDS data
-            st = kvc_stage_tile<REP, KIND>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel, lb);
+            int lane_s = lane;
+            asm volatile("" : "+v"(lane_s));
+            st = kvc_stage_tile<REP, KIND>(a, row, col + 1, lane_s, raw, ops, pack, rows, bias, sel, lb);
         }
     }
 }
@@ -885,8 +901,11 @@ struct KvcSlab {
     static constexpr int WORDS = IS_K ? 64 * K_ROW_WORDS : SLAB * 64 * ESZ / 4;
 };
 
+#ifndef KVC_EXPAND_OCC
+#define KVC_EXPAND_OCC 1
+#endif
 template <int KIND, bool DEQ>
-__global__ void __launch_bounds__(KVC_WG, 4) kvc_expand_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
@@ -942,9 +961,11 @@ __global__ void __launch_bounds__(KVC_WG, 4) kvc_expand_kernel(KvcFusedArgs a)
     for (int it = 0; it < ntiles; it++) {
         const int col = col0 + it;
         const bool more = it + 1 < ntiles;
+        int lane_f = lane;                       // opaque per tile, as in kvc_fused_kernel
+        asm volatile("" : "+v"(lane_f));
         if (more)
             kvc_fetch_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
-                                    __builtin_amdgcn_readlane(bi_bn, it + 1), lane, raw);
+                                    __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
         const float *my_ops = ops + sel * 256;
         const bool fast = fast_loop && st.fits;
         const uint32_t *words = st.fits ? (a.row_words ? rows + lane * a.row_words : pack) : st.gwords;
@@ -1026,7 +1047,11 @@ __global__ void __launch_bounds__(KVC_WG, 4) kvc_expand_kernel(KvcFusedArgs a)
             }
             kvc_wave_sync();
         }
-        if (more) st = kvc_stage_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, lane, raw, ops, pack, rows, bias, sel, lb);
+        if (more) {
+            int lane_s = lane;
+            asm volatile("" : "+v"(lane_s));
+            st = kvc_stage_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, lane_s, raw, ops, pack, rows, bias, sel, lb);
+        }
     }
 }
 
@@ -1190,6 +1215,11 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
         if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
     }
     const dim3 grid = kvc_grid(a.s, rows);
+    static const bool trace_plan = getenv("KVCOMP_TRACE_PLAN") != nullptr;
+    if (trace_plan)
+        fprintf(stderr, "[kvcomp] fused kind %d rep %d: grid %u x %u, lds %zu B (table %d w, payload %d w of %d logical, "
+                "skew %d, rows %d), pair bits %d, tiles per wave %d, rounded %d\n", kind, (int)rep, grid.x, grid.y, lds,
+                a.table_words, a.pack_words, a.pack_logical, a.skew, a.row_words, a.pair_bits, a.s.tiles_per_wave, a.rounded);
     switch (rep) {
         case 1: kvc_launch_fused<1>(kind, a, grid, lds, stream); break;
         case 2: kvc_launch_fused<2>(kind, a, grid, lds, stream); break;
