@@ -702,7 +702,16 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_ke
     const uint32_t mask4 = ((1u << lbits) - 1u) << 2;
     const uint32_t fgroup = lut_g[4], fcheck = lut_g[5];
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
-    const bool dwin = a.double_window != 0 && fgroup >= 4 && n % (2 * (int)fgroup) == 0;   // 64 stream bits per refill
+    // 64 stream bits per refill: `fgroup` symbols from each half.  The main part takes as many refills of
+    // 2 * fgroup symbols as leave a multiple of 8, the rest goes four per half.
+    const bool dwin = a.double_window != 0 && fgroup >= 4 && n % 8 == 0;
+    int n_main = 0;
+    if (dwin) {
+        const int per = 2 * (int)(fgroup > 8u ? 8u : fgroup);
+        int k = n / per;
+        while ((n - k * per) % 8 != 0) k--;
+        n_main = k * per;
+    }
     const uint32_t fe = (uint32_t)(uintptr_t)(kvc_lds_u32 *)s_fentry;  // 0: the table opens the dynamic LDS
 
     // this wave's tiles: T consecutive columns of one tile row
@@ -752,10 +761,13 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_ke
                 constexpr bool SK = decltype(skew_)::value;
                 if (pairs) {
                     kvc_pair_dot<SK, REP>(words, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
-                } else if (dwin && fgroup >= 8 && !fcheck) {
-                    kvc_fast_dot2<8, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
-                } else if (dwin && fgroup >= 4 && fgroup < 8 && !fcheck) {
-                    kvc_fast_dot2<4, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                } else if (dwin && !fcheck) {
+                    if (fgroup >= 8) kvc_fast_dot2<8, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 7) kvc_fast_dot2<7, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 6) kvc_fast_dot2<6, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 5) kvc_fast_dot2<5, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    const int rest = fgroup == 4 ? n : n - n_main;
+                    if (rest) kvc_fast_dot2<4, false, SK, REP>(words, u, fe, mask4, rest, my_ops + (n - rest) * REP, acc, worst);
                 } else if (dwin && fgroup >= 4 && fgroup < 8) {
                     kvc_fast_dot2<4, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else if (fgroup >= 8 && !fcheck) {

@@ -133,7 +133,9 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
         lut[3] = group;
         const bool roomy = s_avg <= 5.5f;
         const bool roomy8 = lmax == 4 && s_avg <= 2.75f;
-        lut[4] = (lmax <= 3 || roomy8) ? 8u : lmax <= 7 ? 4u : roomy ? 4u : 2u;
+        // symbols that a 30-bit window is sure to hold (30 / lmax, at most 8); more where the average code is short
+        // enough for the window to overflow rarely (lut[5] = 1: the kernel checks and falls back)
+        lut[4] = (lmax <= 3 || roomy8) ? 8u : lmax <= 7 ? 30u / lmax : roomy ? 4u : 2u;
         lut[5] = (roomy8 || (lmax > 7 && roomy)) ? 1u : 0u;
         lut[6] = 0;
         lut[7] = 0;
