@@ -234,29 +234,58 @@ __device__ __forceinline__ KvcEmitPlace kvc_emit_place(const KvcEncodeArgs &a, i
     return p;
 }
 
+// The workgroup's copy of the encode table: entries without a usable code become {0, 0} (the count pass has
+// flagged them), and *s_short tells whether every code has at most 8 bits (four then fit one 32-bit group).
+// The caller initialises *s_short to 1 and synchronises before and after.
+__device__ __forceinline__ void kvc_load_code_table(const KvcEncodeArgs &a, uint2 *s_table, uint32_t *s_short, int tid)
+{
+    uint2 e = tid < a.table_entries ? reinterpret_cast<const uint2 *>(a.table)[tid] : make_uint2(0u, 0u);
+    if (e.y > 32u) e = make_uint2(0u, 0u);
+    if (e.y < 32u) e.x &= (1u << e.y) - 1u;               // nothing above the code's own bits
+    s_table[tid] = e;
+    if (e.y > 8u) atomicAnd(s_short, 0u);
+}
+
 // Pack this lane's vector MSB-first at its final position inside the (zeroed) LDS image of the tile payload.
+// The lane's bits pass through a 64-bit accumulator; whenever it holds 32 or more, the oldest 32 leave for the
+// image (what is left above the live bits is never read again, so it is not cleared).  With codes of at most
+// 8 bits the four symbols of a register are first joined into one group of at most 32 bits, which costs a
+// quarter of the accumulator traffic.
 __device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
-                                                const uint2 *s_table, uint32_t *image, uint32_t head)
+                                                const uint2 *s_table, uint32_t *image, uint32_t head, bool short_codes)
 {
     const uint32_t start = lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
     const uint32_t bitpos = (head + start) * 8u;
     uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
     uint64_t acc = 0;
     const int nd = a.vec_len >> 2;
+    auto push = [&](uint32_t bits, uint32_t len) {       // len <= 32, nacc < 32
+        acc = (acc << len) | bits;
+        nacc += len;
+        if (nacc >= 32u) {
+            nacc -= 32u;
+            if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
+            w++;
+        }
+    };
+    if (short_codes) {                                   // wave-uniform
 #pragma unroll
-    for (int j = 0; j < 32; j++) {
-        if (j < nd) {
+        for (int j = 0; j < 32; j++) {
+            if (j < nd) {
+                const uint2 e0 = s_table[v[j] & 0xffu], e1 = s_table[(v[j] >> 8) & 0xffu];
+                const uint2 e2 = s_table[(v[j] >> 16) & 0xffu], e3 = s_table[v[j] >> 24];
+                const uint32_t g = ((((e0.x << e1.y) | e1.x) << e2.y | e2.x) << e3.y) | e3.x;
+                push(g, e0.y + e1.y + e2.y + e3.y);
+            }
+        }
+    } else {
 #pragma unroll
-            for (int k = 0; k < 4; k++) {
-                const uint2 e = s_table[(v[j] >> (8 * k)) & 0xffu];
-                const uint32_t len = e.y > 32u ? 0u : e.y;
-                acc = (acc << len) | e.x;
-                nacc += len;
-                if (nacc >= 32u) {
-                    nacc -= 32u;
-                    if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
-                    w++;
-                    acc &= (1ull << nacc) - 1ull;
+        for (int j = 0; j < 32; j++) {
+            if (j < nd) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint2 e = s_table[(v[j] >> (8 * k)) & 0xffu];
+                    push(e.x, e.y);
                 }
             }
         }
@@ -285,9 +314,12 @@ __device__ __forceinline__ void kvc_write_image(const KvcEncodeArgs &a, const Kv
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a)
 {
     __shared__ uint2 s_table[256];
+    __shared__ uint32_t s_short;
     __shared__ uint32_t s_image[KVC_WAVES_PER_WG][KVC_IMAGE_WORDS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    s_table[tid] = tid < a.table_entries ? reinterpret_cast<const uint2 *>(a.table)[tid] : make_uint2(0u, 0u);
+    if (tid == 0) s_short = 1u;
+    __syncthreads();
+    kvc_load_code_table(a, s_table, &s_short, tid);
     uint32_t *image = s_image[wave];
     __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
@@ -298,7 +330,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a
     uint32_t v[32];
     kvc_load_vector(a, tile, lane, v);
     kvc_wave_lds_sync();
-    kvc_pack_vector(a, tile, lane, v, s_table, image, p.head);
+    kvc_pack_vector(a, tile, lane, v, s_table, image, p.head, s_short != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a, p, lane, image);
 }
@@ -480,8 +512,11 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     __shared__ uint2 s_table[256];
     __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];   // symbols first, then the payload image
     __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];
+    __shared__ uint32_t s_short;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    s_table[tid] = tid < a.e.table_entries ? reinterpret_cast<const uint2 *>(a.e.table)[tid] : make_uint2(0u, 0u);
+    if (tid == 0) s_short = 1u;
+    __syncthreads();
+    kvc_load_code_table(a.e, s_table, &s_short, tid);
     __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
     const KvcEmitPlace p = kvc_emit_place(a.e, tile, tile < a.e.tiles);
@@ -494,7 +529,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
     for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
     kvc_wave_lds_sync();
-    kvc_pack_vector(a.e, tile, lane, v, s_table, image, p.head);
+    kvc_pack_vector(a.e, tile, lane, v, s_table, image, p.head, s_short != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a.e, p, lane, image);
 }
