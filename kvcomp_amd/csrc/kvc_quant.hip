@@ -64,6 +64,48 @@ __device__ __forceinline__ void kvc_quant_store2(const KvcQuantArgs &a, int64_t 
     if (a.xhat) *reinterpret_cast<__half2 *>(a.xhat + i) = __halves2half2(kvc_quant_error_one(v0, g0), kvc_quant_error_one(v1, g1));
 }
 
+// ... of eight adjacent elements of one group (i a multiple of 8; 8- and 16-byte stores)
+template <int GSTEP>   // element k belongs to group g[k * GSTEP]: 0 = one group for all eight, 1 = a group each
+__device__ __forceinline__ void kvc_quant_store8(const KvcQuantArgs &a, int64_t i, const uint4 &raw, const KvcGroupParams *g)
+{
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        v[2 * k] = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
+        v[2 * k + 1] = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+    }
+    if (a.sym) {
+        uint32_t lo = 0, hi = 0;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            lo |= (uint32_t)kvc_quant_one(v[k], g[k * GSTEP]) << (8 * k);
+            hi |= (uint32_t)kvc_quant_one(v[4 + k], g[(4 + k) * GSTEP]) << (8 * k);
+        }
+        *reinterpret_cast<uint2 *>(a.sym + i) = make_uint2(lo, hi);
+    }
+    if (a.xhat) {
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            o[k] = (uint32_t)__half_as_ushort(kvc_quant_error_one(v[2 * k], g[2 * k * GSTEP])) |
+                   ((uint32_t)__half_as_ushort(kvc_quant_error_one(v[2 * k + 1], g[(2 * k + 1) * GSTEP])) << 16);
+        *reinterpret_cast<uint4 *>(a.xhat + i) = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+}
+
+__device__ __forceinline__ void kvc_quant_minmax8(const uint4 &raw, float &mn, float &mx)
+{
+    const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const float v0 = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
+        const float v1 = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+        mn = fminf(mn, fminf(v0, v1));
+        mx = fmaxf(mx, fmaxf(v0, v1));
+    }
+}
+
 __device__ __forceinline__ void kvc_quant_publish(const KvcQuantArgs &a, int64_t g, const KvcGroupParams &gp)
 {
     if (a.scale_f16) a.scale_f16[g] = gp.scale_h;
@@ -100,29 +142,76 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_kernel(KvcQuantArgs 
     }
 }
 
+// The same with eight adjacent channels per thread (16-byte loads, 8-byte symbol stores) for row strides that
+// are a multiple of 8 and 16-byte aligned buffers.
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_channel8_kernel(KvcQuantArgs a)
+{
+    const int64_t stride = a.B * a.H * a.D;
+    const int64_t octs = stride >> 3;
+    const int64_t gid = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
+    if (gid >= a.NB * octs) return;
+    const int64_t nb = gid / octs, c = (gid - nb * octs) * 8;
+    const __half *p = a.x + nb * a.BS * stride + c;
+    float mn[8], mx[8];
+#pragma unroll
+    for (int k = 0; k < 8; k++) { mn[k] = INFINITY; mx[k] = -INFINITY; }
+#pragma unroll 4
+    for (int64_t t = 0; t < a.BS; t++) {
+        const uint4 raw = *reinterpret_cast<const uint4 *>(p + t * stride);
+        const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float v0 = __half2float(__ushort_as_half((unsigned short)(w[k] & 0xffffu)));
+            const float v1 = __half2float(__ushort_as_half((unsigned short)(w[k] >> 16)));
+            mn[2 * k] = fminf(mn[2 * k], v0); mx[2 * k] = fmaxf(mx[2 * k], v0);
+            mn[2 * k + 1] = fminf(mn[2 * k + 1], v1); mx[2 * k + 1] = fmaxf(mx[2 * k + 1], v1);
+        }
+    }
+    KvcGroupParams gp[8];
+    const int64_t g = nb * stride + c;
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        gp[k] = kvc_group_params(mn[k], mx[k], a.eb);
+        kvc_quant_publish(a, g + k, gp[k]);
+    }
+    if (!a.sym && !a.xhat) return;                        // parameters only
+    const int64_t base = nb * a.BS * stride + c;
+#pragma unroll 2
+    for (int64_t t = 0; t < a.BS; t++)
+        kvc_quant_store8<1>(a, base + t * stride, *reinterpret_cast<const uint4 *>(p + t * stride), gp);
+}
+
 // ---- row groups (masks 0xE, 0xC, 0x8): a group is one contiguous run of R elements; one wave per
 // group, min/max by wavefront reduction. -------------------------------------------------------------
-__global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, int64_t R, int64_t groups)
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, int64_t R, int64_t groups, int wide)
 {
     const int lane = threadIdx.x & 63;
     const int64_t g = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
     if (g >= groups) return;
     const __half *p = a.x + g * R;
     float mn = INFINITY, mx = -INFINITY;
-    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
-        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
-        const float v0 = __low2float(v), v1 = __high2float(v);
-        mn = fminf(mn, fminf(v0, v1));
-        mx = fmaxf(mx, fmaxf(v0, v1));
+    if (wide) {                                           // R a multiple of 8, all pointers 16-byte aligned
+        for (int64_t i = 8 * lane; i < R; i += 8 * KVC_WAVE) kvc_quant_minmax8(*reinterpret_cast<const uint4 *>(p + i), mn, mx);
+    } else {
+        for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+            const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+            const float v0 = __low2float(v), v1 = __high2float(v);
+            mn = fminf(mn, fminf(v0, v1));
+            mx = fmaxf(mx, fmaxf(v0, v1));
+        }
     }
     mn = kvc_wave_min(mn);
     mx = kvc_wave_max(mx);
     const KvcGroupParams gp = kvc_group_params(mn, mx, a.eb);
     if (lane == 0) kvc_quant_publish(a, g, gp);
     if (!a.sym && !a.xhat) return;                        // parameters only
-    for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
-        const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
-        kvc_quant_store2(a, g * R + i, __low2float(v), __high2float(v), gp, gp);
+    if (wide) {
+        for (int64_t i = 8 * lane; i < R; i += 8 * KVC_WAVE) kvc_quant_store8<0>(a, g * R + i, *reinterpret_cast<const uint4 *>(p + i), &gp);
+    } else {
+        for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
+            const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
+            kvc_quant_store2(a, g * R + i, __low2float(v), __high2float(v), gp, gp);
+        }
     }
 }
 
@@ -212,13 +301,17 @@ static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t
     a.minmax = nullptr;
     const int64_t stride = B * H * D;
     if (quant_mask == KVC_MASK_CHANNEL) {
-        const int64_t threads = NB * (stride / 2);
-        hipLaunchKernelGGL(kvc_quant_channel_kernel, dim3((unsigned)((threads + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a);
+        const bool wide = stride % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
+        const int64_t threads = NB * (wide ? stride / 8 : stride / 2);
+        const dim3 grid((unsigned)((threads + KVC_WG - 1) / KVC_WG));
+        if (wide) hipLaunchKernelGGL(kvc_quant_channel8_kernel, grid, dim3(KVC_WG), 0, stream, a);
+        else hipLaunchKernelGGL(kvc_quant_channel_kernel, grid, dim3(KVC_WG), 0, stream, a);
     } else if (quant_mask == KVC_MASK_V_TOKEN || quant_mask == KVC_MASK_SIM_TOKEN || quant_mask == KVC_MASK_VECTOR) {
         const int64_t R = quant_mask == KVC_MASK_V_TOKEN ? stride : quant_mask == KVC_MASK_SIM_TOKEN ? H * D : D;
         const int64_t groups = NB * BS * stride / R;
+        const int wide = R % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
         hipLaunchKernelGGL(kvc_quant_row_kernel, dim3((unsigned)((groups + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG)),
-                           dim3(KVC_WG), 0, stream, a, R, groups);
+                           dim3(KVC_WG), 0, stream, a, R, groups, wide);
     } else if (quant_mask == KVC_MASK_K_BLOCK || quant_mask == KVC_MASK_SIM_BLOCK) {
         const int64_t R = quant_mask == KVC_MASK_K_BLOCK ? stride : H * D;
         const int64_t rows = NB * BS * stride / R;

@@ -165,9 +165,16 @@ def test_fused_across_code_length_regimes(eb_k, eb_v):
     print("V lmax", int(s["length"].max()))
 
 
-def _quant_dequant_case(mask, eb):
+@pytest.mark.parametrize("mask", [O.MASK_V_TOKEN, O.MASK_CHANNEL, O.MASK_SIM_TOKEN, O.MASK_VECTOR])
+def test_quant_narrow_rows_bit_exact(mask):
+    """Rows whose length is not a multiple of 8 take the quantizer's two-elements-per-lane kernels instead of the
+    eight-per-lane ones."""
+    _quant_dequant_case(mask, 0.1, geometry=(128, 1, 3, 6))
+
+
+def _quant_dequant_case(mask, eb, geometry=(256, 2, 4, 128)):
     from kvcomp_amd import compute as cp
-    T, B, H, D = 256, 2, 4, 128
+    T, B, H, D = geometry
     x = S.synth_k(T, B, H, D)
     x5 = S.blocked(x, 64)
     _, _, scale, sym, mn = O.quant(S.np16(x5), mask, eb)
