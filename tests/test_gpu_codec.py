@@ -41,7 +41,7 @@ def _make_stream(x_tbhd, is_k, eb, mask, block_size, tree_format=3):
                 code=code, length=length, counts=counts)
 
 
-SHAPES = [(256, 1, 4, 128), (128, 2, 2, 128), (256, 1, 3, 64), (256, 2, 2, 96)]
+SHAPES = [(256, 1, 4, 128), (128, 2, 2, 128), (256, 1, 3, 64), (256, 2, 2, 96), (128, 1, 8, 72), (256, 2, 4, 40)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)

@@ -95,3 +95,29 @@ def test_unsupported_layout_uses_the_symbol_path():
     assert not kvcomp_cuda.store_fused_supported(False, dims_to_mask([4]), 1, 4, 128)      # VectorQuant
     assert not kvcomp_cuda.store_fused_supported(True, dims_to_mask([2, 3, 4]), 1, 4, 128)
     assert kvcomp_cuda.store_fused_supported(True, dims_to_mask([1]), 2, 4, 96)
+
+
+@pytest.mark.parametrize("B,H,D", [(2, 4, 128), (3, 2, 96), (1, 2, 32)])
+def test_fused_store_per_token_and_batch_groups(B, H, D):
+    """V with one scale / minimum per (token, batch entry) (group dimensions [3, 4], mask 0xC): the layout the fused
+    store accepts besides the ones KVCompCtx uses; called directly, compared with the oracle byte for byte."""
+    from kvcomp_amd import kvcomp_cuda as m
+    T, eb, mask = 256, 0.2, O.MASK_SIM_TOKEN
+    assert m.store_fused_supported(False, mask, B, H, D)
+    x = _data(False, T, B, H, D, "gauss", 31)
+    x5 = S.np16(S.blocked(x, 64))
+    _, _, scale, sym, mn = O.quant(x5, mask, eb)
+    counts = np.bincount(sym.ravel(), minlength=256).astype(np.int64)
+    code, length = O.huffman_build(counts)
+    _, enc = O.encode_table(code, length, counts)
+    payload, bi, ti = O.encode_tiles(sym.reshape(T // 128, 128, B, H, D), False, enc, 0, vec_len=128)
+    sizes = m.buffer_sizes(T, B * H * D, False, H, D)
+    bufs = [torch.zeros(n, dtype=torch.uint8, device=DEV) for n in sizes]
+    g_min = torch.zeros(scale.size, dtype=torch.int8, device=DEV)
+    g_scale = torch.zeros(scale.size, dtype=torch.float16, device=DEV)
+    g_enc, g_bi, g_ti = m.store_fused(False, x.to(DEV).contiguous(), mask, eb, torch.from_numpy(enc).to(DEV), g_min, g_scale,
+                                      bufs[0], bufs[1], bufs[2], bufs[3], 0)
+    assert np.array_equal(g_scale.cpu().numpy().view(np.uint16), scale.ravel().view(np.uint16))
+    assert np.array_equal(g_min.cpu().numpy(), mn.ravel())
+    assert np.array_equal(g_ti.cpu().numpy(), ti) and np.array_equal(g_bi.cpu().numpy(), bi)
+    assert np.array_equal(g_enc.cpu().numpy(), payload)
