@@ -94,6 +94,24 @@ int kvc_build_codebook_host(const int64_t *h_counts256, int tree_format, int *sh
                             uint8_t *h_encode_table, int64_t encode_cap, int64_t *encode_bytes,
                             uint8_t *h_decode_tree, int64_t decode_cap, int64_t *decode_bytes);
 
+/* The same on the device, for n_codebooks codebooks in one launch and without a host round trip (the reference
+ * builds every codebook on the host, src/huffman.cpp:99-157, after 256 .item() reads).
+ * kvc_histogram_chunks: one histogram per chunk of chunk_bytes symbols (e.g. the 64-token blocks of a per-block
+ *   codebook), ADDED into d_counts (int64[n_chunks][256]).
+ * kvc_build_codebook_device: d_counts int64[n][256] ->
+ *   d_encode_tables  n x 2048 bytes: the reference's table ({u32 code; u32 length}, entry i = symbol shift + i),
+ *                    zero beyond its (largest - smallest symbol + 1) entries;
+ *   d_decode_trees   n x kvc_codebook_tree_capacity(tree_format) bytes: the reference's node array, followed by
+ *                    childless inner nodes up to the capacity (pass the capacity as tree_bytes to kvc_build_lut);
+ *   d_meta           int32[n][4] = {shift, encode table bytes, decode tree bytes, status}; status 0 = built,
+ *                    1 = fewer than two distinct symbols, 2 = a code exceeds 32 bits, 4 = not representable in the
+ *                    int8 tree (more than 128 nodes or a symbol above 127): then both sizes are 0 and the tables
+ *                    hold no code.  Bytes are identical to what kvc_build_codebook_host returns. */
+int64_t kvc_codebook_tree_capacity(int tree_format);
+int kvc_histogram_chunks(const uint8_t *d_sym, int64_t chunk_bytes, int64_t n_chunks, int64_t *d_counts, void *stream);
+int kvc_build_codebook_device(const int64_t *d_counts, int64_t n_codebooks, int tree_format, uint8_t *d_encode_tables,
+                              uint8_t *d_decode_trees, int32_t *d_meta, void *stream);
+
 /* ---- encode: k_/v_entropy_encode_cuda_export (kernels.cu:919-1011) --------------------------------
  * Writes block_infos (tiles*8 B), thread_infos (tiles*64*2 B) and the payload; *h_total_bytes receives
  * the payload size (the reference returns encoded_data[:total]).  Synchronises the stream before

@@ -32,6 +32,9 @@ _SIGNATURES = {
     "kvc_calculate_buffer_size": [_i64, _i64, _int, _i64, _i64, _i64p],
     "kvc_histogram": [_vp, _i64, _vp, _vp],
     "kvc_build_codebook_host": [_i64p, _int, _intp, _vp, _i64, _i64p, _vp, _i64, _i64p],
+    "kvc_codebook_tree_capacity": [_int],
+    "kvc_histogram_chunks": [_vp, _i64, _i64, _vp, _vp],
+    "kvc_build_codebook_device": [_vp, _i64, _int, _vp, _vp, _vp, _vp],
     "kvc_k_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
     "kvc_v_entropy_encode": [_vp, _i64, _i64, _vp, _i64, _vp, _vp, _vp, _vp, _i64, _u32, _i64, _i64, _i64p, _i64p, _i64p, _vp],
     "kvc_store_fused_supported": [_int, _int, _i64, _i64, _i64],
@@ -64,7 +67,7 @@ _SIGNATURES = {
                              _i64, _i64, _i64, _i64, _f32p, _f32p, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }
-_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_attention_workspace_bytes": _i64,
+_RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_codebook_tree_capacity": _i64, "kvc_attention_workspace_bytes": _i64,
              "kvc_h2_scratch_bytes": _i64}
 
 EXPORTED_SYMBOLS = sorted(list(_SIGNATURES) + ["kvc_last_error"])

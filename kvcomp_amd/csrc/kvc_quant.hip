@@ -401,11 +401,15 @@ extern "C" int kvc_dequant(const uint8_t *d_sym, const int8_t *d_min_i8, const v
 // One counter per (bin, lane & 31): counter (bin, c) lives in LDS bank c, so the lanes of a half wave never
 // collide on a bank, whatever the symbol distribution (KV symbols are heavily skewed: most lanes add to the
 // same one or two bins).  Only lanes l and l + 32, and the workgroup's other waves, share a counter.
+// blockIdx.y selects one of several equal chunks of `n` symbols, `chunk_stride` bytes apart, each with its own
+// 256 counters.
 __global__ void __launch_bounds__(KVC_WG) kvc_histogram_kernel(const uint8_t *__restrict__ sym, int64_t n,
-                                                               unsigned long long *__restrict__ counts)
+                                                               unsigned long long *__restrict__ counts, int64_t chunk_stride)
 {
     __shared__ uint32_t s_bins[256 * 32];
     const int tid = threadIdx.x, col = tid & 31;
+    sym += (int64_t)blockIdx.y * chunk_stride;
+    counts += (int64_t)blockIdx.y * 256;
     for (int i = tid; i < 256 * 32; i += KVC_WG) s_bins[i] = 0;
     __syncthreads();
     // bytes in front of the first 16-byte boundary, whole 16-byte groups, bytes after the last one
@@ -448,7 +452,23 @@ extern "C" int kvc_histogram(const uint8_t *d_sym, int64_t n, int64_t *d_counts,
     if (wgs > 4096) wgs = 4096;
     KVC_REQUIRE(n / wgs < (1ll << 31), "input too large for 32-bit workgroup counters");
     hipLaunchKernelGGL(kvc_histogram_kernel, dim3((unsigned)wgs), dim3(KVC_WG), 0, stream, d_sym, n,
-                       reinterpret_cast<unsigned long long *>(d_counts));
+                       reinterpret_cast<unsigned long long *>(d_counts), (int64_t)0);
+    return kvc_check_hip(hipGetLastError(), "kvc_histogram_kernel launch");
+}
+
+// d_counts[c * 256 + s] += occurrences of symbol s among d_sym[c * chunk_bytes .. (c + 1) * chunk_bytes)
+extern "C" int kvc_histogram_chunks(const uint8_t *d_sym, int64_t chunk_bytes, int64_t n_chunks, int64_t *d_counts, void *stream_)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    KVC_REQUIRE(chunk_bytes >= 0 && n_chunks >= 0 && n_chunks <= 65535, "bad chunk geometry (%lld chunks of %lld bytes)",
+                (long long)n_chunks, (long long)chunk_bytes);
+    if (chunk_bytes == 0 || n_chunks == 0) return 0;
+    int64_t wgs = (chunk_bytes / 16 + KVC_WG * 8 - 1) / (KVC_WG * 8);
+    if (wgs < 1) wgs = 1;
+    if (wgs > 4096) wgs = 4096;
+    KVC_REQUIRE(chunk_bytes / wgs < (1ll << 31), "chunk too large for 32-bit workgroup counters");
+    hipLaunchKernelGGL(kvc_histogram_kernel, dim3((unsigned)wgs, (unsigned)n_chunks), dim3(KVC_WG), 0, stream, d_sym,
+                       chunk_bytes, reinterpret_cast<unsigned long long *>(d_counts), chunk_bytes);
     return kvc_check_hip(hipGetLastError(), "kvc_histogram_kernel launch");
 }
 

@@ -108,6 +108,36 @@ def build_codebook_from_counts(counts: torch.Tensor, tree_format: int = TREE_I8)
     return shift.value, enc[:eb.value].clone(), dec[:db.value].clone()
 
 
+def symbol_counts_chunks(symbols: torch.Tensor, n_chunks: int) -> torch.Tensor:
+    """One 256-bin histogram per equal chunk of a contiguous device uint8 tensor (e.g. per 64-token block), as a
+    device int64 tensor [n_chunks, 256]; nothing waits for the host."""
+    _dev_u8(symbols, "symbols")
+    _require(symbols.is_contiguous() and n_chunks > 0 and symbols.numel() % n_chunks == 0, "symbols must split into equal chunks")
+    with torch.cuda.device(symbols.device):
+        counts = torch.zeros(n_chunks, 256, dtype=torch.int64, device=symbols.device)
+        check(_lib.lib().kvc_histogram_chunks(_ptr(symbols), symbols.numel() // n_chunks, n_chunks, _ptr(counts), _stream(symbols)))
+    return counts
+
+
+def build_codebook_device(counts: torch.Tensor, tree_format: int = TREE_I8):
+    """build_codebook (src/huffman.cpp:99-157) for every row of a device int64 tensor [n, 256], on the device.
+    Returns device tensors (encode tables uint8 [n, 2048], decode trees uint8 [n, capacity], meta int32 [n, 4] =
+    {shift, encode table bytes, decode tree bytes, status}); rows with a non-zero status hold no code (1: fewer than
+    two symbols, 2: a code beyond 32 bits, 4: not representable in the int8 tree).  The trees are padded to their
+    capacity, which is the `tree_bytes` to give kvc_build_lut."""
+    _require(counts.is_cuda and counts.dtype == torch.int64 and counts.dim() == 2 and counts.shape[1] == 256 and
+             counts.is_contiguous(), "counts must be a contiguous device int64 tensor [n, 256]")
+    n = counts.shape[0]
+    cap = int(_lib.lib().kvc_codebook_tree_capacity(tree_format))
+    _require(cap > 0, "unknown tree format")
+    with torch.cuda.device(counts.device):
+        enc = torch.empty(n, 2048, dtype=torch.uint8, device=counts.device)
+        trees = torch.empty(n, cap, dtype=torch.uint8, device=counts.device)
+        meta = torch.empty(n, 4, dtype=torch.int32, device=counts.device)
+        check(_lib.lib().kvc_build_codebook_device(_ptr(counts), n, tree_format, _ptr(enc), _ptr(trees), _ptr(meta), _stream(counts)))
+    return enc, trees, meta
+
+
 def _entropy_encode(is_k, input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
                     base_global_offset, head_num, head_dim):
     for t, n in ((input, "input"), (encode_code_book, "encode_code_book"), (block_infos, "block_infos"),
