@@ -131,6 +131,15 @@ __device__ __forceinline__ uint32_t kvc_refill_address(uint32_t stage_base, uint
 }
 constexpr int KVC_LDS_SLACK_WORDS = 48;
 
+// Rounded mode: RN16((sym + min) * scale) as the reference's dequantizer computes it (sym + min exactly, one
+// rounding of the product).  Both steps are fp16 instructions: the sum of two small integers is exact in fp16
+// and an fp16 multiplication rounds the exact product once.  `ms` = {min, scale} as two fp16 in one word.
+__device__ __forceinline__ float kvc_rounded_value(__half sym, uint32_t ms)
+{
+    const __half mn = __ushort_as_half((unsigned short)(ms & 0xffffu)), sc = __ushort_as_half((unsigned short)(ms >> 16));
+    return __half2float(__hmul(__hadd(sym, mn), sc));
+}
+
 // -- slow path ----------------------------------------------------------------------------------------
 // One symbol per refill; table and long-code list in global memory; words from LDS (staged, bit-reversed)
 // or from global memory (raw, bounds-checked word by word).
@@ -175,10 +184,10 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
         }
         const float f = (float)sym;
         if (rounded) {
-            const float *o = ops + i * (REP + 2);
-            const float v = __half2float(__float2half_rn((f + o[0]) * o[1]));
+            const float *o = ops + i * (REP + 1);
+            const float v = kvc_rounded_value(__float2half_rn(f), __float_as_uint(o[0]));
 #pragma unroll
-            for (int r = 0; r < REP; r++) acc.v[r] = fmaf(v, o[2 + r], acc.v[r]);
+            for (int r = 0; r < REP; r++) acc.v[r] = fmaf(v, o[1 + r], acc.v[r]);
         } else {
 #pragma unroll
             for (int r = 0; r < REP; r++) acc.v[r] = fmaf(f, ops[i * REP + r], acc.v[r]);
@@ -305,31 +314,32 @@ __device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t &u
 }
 
 // Rounded mode: the dequantized value is rounded to fp16 before the multiplication (see KvcFusedArgs::rounded).
-// Four symbols per refill (codes of at most 7 bits); the element's {min, scale, weights} come from one address
-// for the whole wave.
+// 64 stream bits per refill, four symbols from each half (codes of at most 7 bits).  The table entries carry the
+// symbol as fp16 in their upper half (and the length in the lowest byte); element i's {min, scale} (two fp16 in
+// one word) and weights come from one address for the whole wave.
 template <bool SKEW, int REP>
 __device__ __forceinline__ void kvc_rounded_dot(const uint32_t *stage, uint32_t &u, uint32_t fentry_base, uint32_t mask4,
                                                 int n, const float *ops, float (&acc)[REP])
 {
-    constexpr int OPS = REP + 2;
+    constexpr int OPS = REP + 1;
     const uint32_t sbase = (uint32_t)(uintptr_t)(const kvc_lds_word *)stage;
-    for (int i = 0; i < n; i += 4) {
+    for (int i = 0; i < n; i += 8) {
         const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
-        const uint32_t w0 = wp[0], w1 = wp[1];
-        uint32_t R = __builtin_amdgcn_alignbit(w1, w0, u);
-        uint32_t es = 0;
-        kvc_static_for<4>([&](auto g_) {
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0;
+        kvc_static_for<8>([&](auto g_) {
             constexpr int g = decltype(g_)::value;
+            if (g == 4) R = __builtin_amdgcn_alignbit(hi, lo, es);        // at most 28 bits consumed so far
             const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
-            R = __builtin_amdgcn_alignbit(R, R, e);
-            es += e;
-            const float f = __uint_as_float(e & 0xffffff00u);              // the symbol, exactly
+            if (g != 3 && g != 7) R = __builtin_amdgcn_alignbit(R, R, e);
+            es += e & 0xffu;
             const float *o = ops + (i + g) * OPS;
-            const float v = __half2float(__float2half_rn((f + o[0]) * o[1]));
+            const float v = kvc_rounded_value(__ushort_as_half((unsigned short)(e >> 16)), __float_as_uint(o[0]));
 #pragma unroll
-            for (int r = 0; r < REP; r++) acc[r] = fmaf(v, o[2 + r], acc[r]);
+            for (int r = 0; r < REP; r++) acc[r] = fmaf(v, o[1 + r], acc[r]);
         });
-        u += es & 0xffu;
+        u += es;
     }
 }
 
@@ -594,11 +604,11 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
             const float sc = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
             const float mn = (float)raw.mn[s][half];
             if (a.rounded) {                             // wave-uniform
-                float *o = ops + (s * 128 + i) * (REP + 2);
-                o[0] = mn;
-                o[1] = sc;
+                float *o = ops + (s * 128 + i) * (REP + 1);
+                const uint32_t mn_h = __half_as_ushort(__float2half_rn(mn));                  // exact
+                o[0] = __uint_as_float(mn_h | ((live ? (uint32_t)raw.sc[s][half] : 0u) << 16));
 #pragma unroll
-                for (int r = 0; r < REP; r++) o[2 + r] = wgt[r][half];
+                for (int r = 0; r < REP; r++) o[1 + r] = wgt[r][half];
                 continue;
             }
 #pragma unroll
@@ -658,7 +668,7 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_ke
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int D = a.head_dim;
-    const int ops_per_elem = a.rounded ? REP + 2 : REP;
+    const int ops_per_elem = a.rounded ? REP + 1 : REP;
     const int per_wave = SLOTS * 128 * ops_per_elem + a.pack_words + KVC_WAVE * a.row_words;
     uint32_t *s_fentry = smem;
     float *ops = reinterpret_cast<float *>(smem + a.table_words + wave * per_wave);
@@ -692,6 +702,13 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_ke
             smem[2 * idx + 1] = e1;
         }
         __syncthreads();
+    } else if (fast_book && a.rounded) {
+        // the symbol as fp16 in the upper half of the entry, the length in its lowest byte
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) {
+            const uint32_t e = fentry(i);
+            const uint32_t sym_h = __half_as_ushort(__float2half_rn(__uint_as_float(e & 0xffffff00u)));
+            s_fentry[i] = (sym_h << 16) | (e & 0xffu);
+        }
     } else if (fast_book) {
         for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) s_fentry[i] = fentry(i);
     }
@@ -1085,7 +1102,8 @@ static void kvc_launch_fused(int kind, const KvcFusedArgs &a, dim3 grid, size_t 
 // longest lane stream); without them from twice the payload's means.  Tiles that do not fit are decoded
 // from global memory, so the sizes only affect speed.  Everything stays within 64 KiB per workgroup.
 static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_bytes, int64_t tiles,
-                           int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t extra_words = 0)
+                           int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t extra_words = 0,
+                           bool allow_pairs = true)
 {
     const int force_rows = kvc_option(KVC_OPT_FUSED_ROWS);   // 0 / 1 overrides the choice below
     a.table_words = 1 << ((max_code_bits >= 1 && max_code_bits <= KVC_LUT_MAX_BITS) ? max_code_bits : KVC_LUT_MAX_BITS);
@@ -1097,7 +1115,7 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     a.expand = 0;
     a.out_words = 0;
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
-    if (extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
+    if (allow_pairs && extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
         a.pair_bits = 2 * max_code_bits;
         if (a.table_words < (2 << a.pair_bits)) a.table_words = 2 << a.pair_bits;
     }
@@ -1219,8 +1237,8 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
     const int kind = is_k ? 0 : (a.scores ? 2 : 0) + slots;
     const int rounded = kvc_option(KVC_OPT_FUSED_ROUNDED) != 0;
-    const size_t lds = kvc_plan_lds(a, slots, rounded ? (int)rep + 2 : (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
-                                    max_stream_bytes, rounded ? 0 : max_code_bits);
+    const size_t lds = kvc_plan_lds(a, slots, rounded ? (int)rep + 1 : (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
+                                    max_stream_bytes, max_code_bits, 0, !rounded);
     a.rounded = rounded;
     a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
     KvcTimer timer(elapsed_ms, stream);
