@@ -333,13 +333,13 @@ __device__ __forceinline__ void kvc_rounded_dot(const uint32_t *stage, uint32_t 
             if (g == 4) R = __builtin_amdgcn_alignbit(hi, lo, es);        // at most 28 bits consumed so far
             const uint32_t e = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fentry_base);
             if (g != 3 && g != 7) R = __builtin_amdgcn_alignbit(R, R, e);
-            es += e & 0xffu;
+            es += e;                                                       // only the lowest byte is read below
             const float *o = ops + (i + g) * OPS;
             const float v = kvc_rounded_value(__ushort_as_half((unsigned short)(e >> 16)), __float_as_uint(o[0]));
 #pragma unroll
             for (int r = 0; r < REP; r++) acc[r] = fmaf(v, o[1 + r], acc[r]);
         });
-        u += es;
+        u += es & 0xffu;
     }
 }
 
@@ -565,12 +565,12 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
         if (s == 1 && !straddles) continue;                    // no lane of this tile belongs to a second head
         const bool live = KIND != 0 || 2 * lane < D;
         if (EXPAND == 1) continue;
-        if (EXPAND == 2) {                           // element i of slot s -> {scale, min} at ops[(s * 128 + i) * 2]
+        if (EXPAND == 2) {                           // element i of slot s -> {min, scale} as two fp16 at ops[s * 128 + i]
 #pragma unroll
             for (int half = 0; half < 2; half++) {
                 const int i = 2 * lane + half;
-                ops[(s * 128 + i) * 2] = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
-                ops[(s * 128 + i) * 2 + 1] = (float)raw.mn[s][half];
+                const uint32_t mn_h = __half_as_ushort(__float2half_rn((float)raw.mn[s][half]));   // exact
+                ops[s * 128 + i] = __uint_as_float(mn_h | ((live ? (uint32_t)raw.sc[s][half] : 0u) << 16));
             }
             continue;
         }
@@ -944,7 +944,7 @@ __global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcF
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int D = a.head_dim;
-    const int ops_words = DEQ ? SLOTS * 128 * 2 : 0;
+    const int ops_words = DEQ ? SLOTS * 128 : 0;
     const int per_wave = ops_words + a.pack_words + KVC_WAVE * a.row_words + a.out_words;
     uint32_t *s_fentry = smem;
     float *ops = reinterpret_cast<float *>(smem + a.table_words + wave * per_wave);
@@ -958,8 +958,11 @@ __global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcF
     const bool fast_book = nlong == 0 && lbits <= (uint32_t)KVC_LUT_MAX_BITS && (1u << lbits) <= (uint32_t)a.table_words;
     if (fast_book)
         for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) {
-            const uint32_t e = lut_g[KVC_LUT_FENTRY_OFFSET + i];
-            s_fentry[i] = (e & 0xffu) > lbits ? (e & ~0xffu) | lbits : e;
+            uint32_t e = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+            e = (e & 0xffu) > lbits ? (e & ~0xffu) | lbits : e;
+            // dequantizing: the symbol as fp16 in the upper half of the entry, the length in its lowest byte
+            if (DEQ) e = ((uint32_t)__half_as_ushort(__float2half_rn(__uint_as_float(e & 0xffffff00u))) << 16) | (e & 0xffu);
+            s_fentry[i] = e;
         }
     if (lane < KVC_PACK_LEAD) pack[lane] = 0;
     if (a.row_words) rows[lane * a.row_words] = 0;
@@ -995,19 +998,21 @@ __global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcF
         if (more)
             kvc_fetch_tile<1, KIND, DEQ ? 2 : 1>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
                                     __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
-        const float *my_ops = ops + sel * 256;
+        const float *my_ops = ops + sel * 128;
         const bool fast = fast_loop && st.fits;
         const uint32_t *words = st.fits ? (a.row_words ? rows + lane * a.row_words : pack) : st.gwords;
         const uint32_t nw = st.fits ? (uint32_t)(a.row_words ? a.row_words : a.pack_logical) : st.gnwords;
         const bool skew = st.fits && !a.row_words && a.skew;
         uint32_t u = st.fits ? st.u0 : st.gpos;                 // fast: lb bits before the code; slow: at the code
         if (st.fits && !fast) u += lb;
-        // the value of element i: the symbol itself, or (symbol + min_i) * scale_i rounded to fp16
-        auto value = [&](int i, uint32_t e) -> uint32_t {
+        // the value of element i: the symbol itself, or RN16((symbol + min_i) * scale_i) (an exact fp16 sum and one
+        // fp16 multiplication).  FAST: e is a table entry of this kernel; otherwise the symbol as an fp32 pattern.
+        auto value = [&](int i, uint32_t e, bool from_table) -> uint32_t {
             if (DEQ) {
-                const float f = __uint_as_float(e & 0xffffff00u);          // the symbol, exactly
-                const float2 sm = *reinterpret_cast<const float2 *>(my_ops + 2 * i);
-                return (uint32_t)__half_as_ushort(__float2half_rn((f + sm.y) * sm.x));
+                const __half sym = from_table ? __ushort_as_half((unsigned short)(e >> 16)) : __float2half_rn(__uint_as_float(e));
+                const uint32_t ms = __float_as_uint(my_ops[i]);
+                const __half mn = __ushort_as_half((unsigned short)(ms & 0xffffu)), sc = __ushort_as_half((unsigned short)(ms >> 16));
+                return (uint32_t)__half_as_ushort(__hmul(__hadd(sym, mn), sc));
             }
             return (uint32_t)__uint_as_float(e);                           // the low mantissa bits add less than one
         };
@@ -1017,7 +1022,7 @@ __global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcF
         auto put = [&](int i, auto g_, uint32_t e) {
             constexpr int g = decltype(g_)::value;
             constexpr int PER = 4 / S::ESZ;                                // elements per word
-            const uint32_t v = value(i + g, e);
+            const uint32_t v = value(i + g, e, true);
             if (IS_K) {
                 cur = (g % PER == 0) ? v : cur | (v << (8 * S::ESZ * (g % PER)));
                 if (g % PER == PER - 1)
@@ -1029,7 +1034,7 @@ __global__ void __launch_bounds__(KVC_WG, KVC_EXPAND_OCC) kvc_expand_kernel(KvcF
         // slow loop: one element at a time
         auto put1 = [&](int i, uint32_t e) {
             const int j = i & (S::SLAB - 1);
-            slab[IS_K ? lane * (S::K_ROW_WORDS * 4 / S::ESZ) + j : j * KVC_WAVE + lane] = (elem)value(i, e);
+            slab[IS_K ? lane * (S::K_ROW_WORDS * 4 / S::ESZ) + j : j * KVC_WAVE + lane] = (elem)value(i, e, false);
         };
         for (int i0 = 0; i0 < n; i0 += S::SLAB) {
             const int len = n - i0 < S::SLAB ? n - i0 : S::SLAB;
@@ -1303,7 +1308,7 @@ int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_t
     const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
     const int out_words = is_k ? (deq ? KvcSlab<true, true>::WORDS : KvcSlab<true, false>::WORDS)
                                : (deq ? KvcSlab<false, true>::WORDS : KvcSlab<false, false>::WORDS);
-    const size_t lds = kvc_plan_lds(a, slots, deq ? 2 : 0, encoded_bytes, rows * a.s.cols, 0, 0, 0, out_words);
+    const size_t lds = kvc_plan_lds(a, slots, deq ? 1 : 0, encoded_bytes, rows * a.s.cols, 0, 0, 0, out_words);
     a.expand = deq ? 2 : 1;
     a.out_words = out_words;
     a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
