@@ -366,9 +366,9 @@ def test_fused_k_window_groupings(nsym, expect_lmax):
     assert np.abs(out.float().cpu().numpy() - ref).max() <= 1e-3 * np.abs(ref).max()
 
 
-@pytest.mark.parametrize("D", [64, 96, 128, 72])
+@pytest.mark.parametrize("D,rep", [(64, 1), (96, 1), (128, 1), (72, 1), (128, 4), (96, 2), (64, 8)])
 @pytest.mark.parametrize("nsym,expect_lmax", [(12, 4), (24, 5), (40, 6), (100, 7)])
-def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D):
+def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D, rep):
     """Exactly uniform alphabets give codes of 4 to 7 bits, for which a 30-bit half window is sure to hold 7, 6, 5
     and 4 symbols: the kernel decodes 14, 12, 10 or 8 symbols per refill and finishes a vector whose length is not
     a multiple of that with refills of 8 (head_dim 64, 72, 96 and 128; V vectors hold 128 symbols)."""
@@ -387,9 +387,9 @@ def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D):
     gs = O.group_shape(sym.shape, O.MASK_CHANNEL)
     mn = rng.integers(-(nsym // 2) - 1, 0, size=gs).astype(np.int8)
     scale = rng.uniform(0.01, 0.2, size=gs).astype(np.float16)
-    q = S.synth_q(B, H, D)
+    q = S.synth_q(B, H * rep, D)
     ref = O.fused_k(sym.reshape(T, B, H, D), mn, scale, O.MASK_CHANNEL, 64, S.np16(q))
-    out = torch.zeros(B, H, T, dtype=torch.float16, device=DEV)
+    out = torch.zeros(B, H * rep, T, dtype=torch.float16, device=DEV)
     m.k_decode_and_mat_vec_mul_cuda_export(dec.to(DEV), g_bi, g_ti, g_enc, _dev(mn.ravel()),
                                            _dev(scale.ravel().view(np.uint16), torch.float16), q.to(DEV), out, H, D,
                                            tree_format=fmt)
@@ -403,9 +403,9 @@ def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D):
         gsv = O.group_shape(symv.shape, O.MASK_V_TOKEN)
         mnv = rng.integers(-(nsym // 2) - 1, 0, size=gsv).astype(np.int8)
         scv = rng.uniform(0.01, 0.2, size=gsv).astype(np.float16)
-        p = S.synth_p(B, H, T)
+        p = S.synth_p(B, H * rep, T)
         refv = O.fused_v(symv.reshape(T, B, H, D), mnv, scv, O.MASK_V_TOKEN, 128, S.np16(p))
-        part = torch.zeros(T // 128, B, H, D, dtype=torch.float16, device=DEV)
+        part = torch.zeros(T // 128, B, H * rep, D, dtype=torch.float16, device=DEV)
         m.v_decode_and_mat_vec_mul_cuda_export(dec.to(DEV), v_bi, v_ti, v_enc, _dev(mnv.ravel()),
                                                _dev(scv.ravel().view(np.uint16), torch.float16), p.to(DEV), part, H, D,
                                                tree_format=fmt)
