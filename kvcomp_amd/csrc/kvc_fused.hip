@@ -1471,7 +1471,12 @@ kvc_tail_values_kernel(const __half *__restrict__ tail, const float *__restrict_
 }
 
 // out[b, hq, :] from `groups` partials; one workgroup of 16 waves per (b, hq), wave w takes groups w, w + 16, ...
+// Each wave sums its groups relative to a maximum of its own -- U groups at a time, all their loads issued
+// together (indices past the end are clamped and weighted zero, so nothing branches around a load) -- and the
+// waves' sums are brought to the common maximum when they are merged: a 32k-token context is one round trip to
+// memory and one barrier.
 constexpr int KVC_COMBINE_WAVES = 16;
+template <int U>
 __global__ void __launch_bounds__(KVC_COMBINE_WAVES * KVC_WAVE)
 kvc_attention_combine_kernel(const float *__restrict__ part, const float *__restrict__ ml, int64_t groups,
                              int64_t bhq_count, int D, float *__restrict__ out)
@@ -1481,44 +1486,48 @@ kvc_attention_combine_kernel(const float *__restrict__ part, const float *__rest
     __shared__ float s_den[KVC_COMBINE_WAVES];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int64_t bhq = blockIdx.x;
-    // global maximum
-    float m = -INFINITY;
-    for (int64_t g = threadIdx.x; g < groups; g += KVC_COMBINE_WAVES * KVC_WAVE) m = fmaxf(m, ml[(g * bhq_count + bhq) * 2]);
-    m = kvc_wave_fmax_dpp(m);
-    if (lane == 0) s_max[wave] = m;
-    __syncthreads();
-    float M = s_max[0];
-#pragma unroll
-    for (int w = 1; w < KVC_COMBINE_WAVES; w++) M = fmaxf(M, s_max[w]);
-    float n0 = 0.f, n1 = 0.f, den = 0.f;
-    constexpr int U = 4;                                  // groups in flight per wave
+    const int d0 = lane < D ? lane : 0, d1 = lane + 64 < D ? lane + 64 : 0;
+    float M = -INFINITY, n0 = 0.f, n1 = 0.f, den = 0.f;   // this wave's running maximum and its sums relative to it
     for (int64_t g0 = wave; g0 < groups; g0 += U * KVC_COMBINE_WAVES) {
         float mg[U], lg[U], p0[U], p1[U];
 #pragma unroll
         for (int u = 0; u < U; u++) {
             const int64_t g = g0 + u * KVC_COMBINE_WAVES;
-            mg[u] = -INFINITY;
-            lg[u] = p0[u] = p1[u] = 0.f;
-            if (g < groups) {
-                const float *mlp = ml + (g * bhq_count + bhq) * 2;
-                const float *pp = part + (g * bhq_count + bhq) * D;
-                mg[u] = mlp[0];
-                lg[u] = mlp[1];
-                if (lane < D) p0[u] = pp[lane];
-                if (lane + 64 < D) p1[u] = pp[lane + 64];
-            }
+            const int64_t gc = g < groups ? g : groups - 1;
+            const float *mlp = ml + (gc * bhq_count + bhq) * 2;
+            const float *pp = part + (gc * bhq_count + bhq) * D;
+            mg[u] = g < groups ? mlp[0] : -INFINITY;
+            lg[u] = mlp[1];
+            p0[u] = pp[d0];
+            p1[u] = pp[d1];
+        }
+        float mb = mg[0];
+#pragma unroll
+        for (int u = 1; u < U; u++) mb = fmaxf(mb, mg[u]);
+        if (mb > M) {                                     // wave-uniform; rescale what has been summed so far
+            const float f = __expf(M - mb);               // exp(-inf) = 0 the first time
+            n0 *= f;
+            n1 *= f;
+            den *= f;
+            M = mb;
         }
 #pragma unroll
         for (int u = 0; u < U; u++) {
-            const float f = __expf(mg[u] - M);             // exp(-inf) = 0 for the slots past the end
+            const float f = __expf(mg[u] - M);            // 0 for the slots past the end (M is finite here)
             den += f * lg[u];
             n0 += f * p0[u];
             n1 += f * p1[u];
         }
     }
-    s_num[wave][lane] = n0;
-    s_num[wave][lane + 64] = n1;
-    if (lane == 0) s_den[wave] = den;
+    if (lane == 0) s_max[wave] = M;
+    __syncthreads();
+    float Mall = s_max[0];
+#pragma unroll
+    for (int w = 1; w < KVC_COMBINE_WAVES; w++) Mall = fmaxf(Mall, s_max[w]);
+    const float fw = M == -INFINITY ? 0.f : __expf(M - Mall);          // a wave without groups contributes nothing
+    s_num[wave][lane] = lane < D ? n0 * fw : 0.f;
+    s_num[wave][lane + 64] = lane + 64 < D ? n1 * fw : 0.f;
+    if (lane == 0) s_den[wave] = den * fw;
     __syncthreads();
     if (threadIdx.x < D) {
         const int d = threadIdx.x;
@@ -1618,8 +1627,15 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
                            part + g * batch * q_heads * head_dim, ml + g * batch * q_heads * 2, v->tokens, v->tail_tokens,
                            (int)batch, (int)kv_heads, rep, (int)head_dim);
     }
-    hipLaunchKernelGGL(kvc_attention_combine_kernel, dim3((unsigned)(batch * q_heads)), dim3(KVC_COMBINE_WAVES * KVC_WAVE), 0, stream, part, ml,
-                       p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+    // groups in flight per wave: what one pass over a wave's share needs, at most 16
+    const dim3 cgrid((unsigned)(batch * q_heads)), cblock(KVC_COMBINE_WAVES * KVC_WAVE);
+    const int64_t per_wave = (p.groups + KVC_COMBINE_WAVES - 1) / KVC_COMBINE_WAVES;
+    if (per_wave <= 4)
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<4>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+    else if (per_wave <= 8)
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<8>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+    else
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<16>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
     KVC_HIP(hipGetLastError());
     return timer.finish();
 }
