@@ -1445,28 +1445,69 @@ kvc_tail_scores_kernel(const __half *__restrict__ tail, const __half *__restrict
     }
 }
 
-// The tail tokens [t0, t0 + n) as one more group: one workgroup per (b, hq); thread d accumulates channel d.
-__global__ void __launch_bounds__(128)
+// The tail tokens [t0, t0 + n) as one more group: one workgroup of four waves per (b, hq).  The tokens are taken
+// 256 at a time: every thread turns one score into a weight (against the group's maximum, found first), then wave w
+// adds tokens w, w + 4, ... of the chunk, lane l holding channels 2l and 2l + 1 (one coalesced row read per token).
+constexpr int KVC_TAIL_WAVES = 4;
+__global__ void __launch_bounds__(KVC_TAIL_WAVES * KVC_WAVE)
 kvc_tail_values_kernel(const __half *__restrict__ tail, const float *__restrict__ scores, int64_t scores_stride,
                        float sm_scale, float *__restrict__ part, float *__restrict__ ml, int64_t t0, int64_t n,
                        int batch, int kv_heads, int rep, int D)
 {
+    constexpr int CHUNK = KVC_TAIL_WAVES * KVC_WAVE;
+    __shared__ float s_red[KVC_TAIL_WAVES];
+    __shared__ float s_w[CHUNK];
+    __shared__ float s_acc[KVC_TAIL_WAVES][2 * KVC_WAVE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int hq = blockIdx.x % (kv_heads * rep), b = blockIdx.x / (kv_heads * rep);
     const int h = hq / rep;
     const float *sp = scores + ((int64_t)b * kv_heads * rep + hq) * scores_stride + t0;
+    // the group's maximum
     float m = -INFINITY;
-    for (int64_t t = 0; t < n; t++) m = fmaxf(m, sp[t] * sm_scale);
-    float l = 0.f, acc = 0.f;
-    const int d = threadIdx.x;
-    for (int64_t t = 0; t < n; t++) {
-        const float w = __expf(sp[t] * sm_scale - m);
+    for (int64_t t = tid; t < n; t += CHUNK) m = fmaxf(m, sp[t] * sm_scale);
+    m = kvc_wave_fmax_dpp(m);
+    if (lane == 0) s_red[wave] = m;
+    __syncthreads();
+    m = s_red[0];
+#pragma unroll
+    for (int w = 1; w < KVC_TAIL_WAVES; w++) m = fmaxf(m, s_red[w]);
+    float l = 0.f, acc0 = 0.f, acc1 = 0.f;
+    const bool live = 2 * lane < D;
+    const int64_t row = (int64_t)batch * kv_heads * D;                  // halves per token
+    const __half *vp = tail + ((int64_t)b * kv_heads + h) * D + (live ? 2 * lane : 0);
+    for (int64_t c0 = 0; c0 < n; c0 += CHUNK) {
+        const int64_t t = c0 + tid;
+        const float w = t < n ? __expf(sp[t] * sm_scale - m) : 0.f;
+        __syncthreads();                                               // the previous chunk's weights have been used
+        s_w[tid] = w;
         l += w;
-        if (d < D) acc += w * __half2float(tail[((t * batch + b) * kv_heads + h) * D + d]);
+        __syncthreads();
+        const int len = (int)(n - c0 < CHUNK ? n - c0 : CHUNK);
+        for (int k = wave; k < len; k += KVC_TAIL_WAVES) {
+            const float wk = s_w[k];
+            const __half2 v = *reinterpret_cast<const __half2 *>(vp + (c0 + k) * row);
+            acc0 += wk * __low2float(v);
+            acc1 += wk * __high2float(v);
+        }
     }
-    if (d < D) part[((int64_t)b * kv_heads * rep + hq) * D + d] = acc;
-    if (d == 0) {
+    l = kvc_wave_sum_dpp(l);
+    __syncthreads();
+    if (lane == 0) s_red[wave] = l;
+    s_acc[wave][2 * lane] = acc0;
+    s_acc[wave][2 * lane + 1] = acc1;
+    __syncthreads();
+    if (tid < D) {
+        float a = 0.f;
+#pragma unroll
+        for (int w = 0; w < KVC_TAIL_WAVES; w++) a += s_acc[w][tid];
+        part[((int64_t)b * kv_heads * rep + hq) * D + tid] = a;
+    }
+    if (tid == 0) {
+        float lsum = 0.f;
+#pragma unroll
+        for (int w = 0; w < KVC_TAIL_WAVES; w++) lsum += s_red[w];
         ml[((int64_t)b * kv_heads * rep + hq) * 2] = m;
-        ml[((int64_t)b * kv_heads * rep + hq) * 2 + 1] = l;
+        ml[((int64_t)b * kv_heads * rep + hq) * 2 + 1] = lsum;
     }
 }
 
@@ -1622,7 +1663,7 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
     }
     if (v->tail_tokens) {
         const int64_t g = v->tokens / KVC_V_TOKENS;
-        hipLaunchKernelGGL(kvc_tail_values_kernel, dim3((unsigned)(batch * q_heads)), dim3(128), 0, stream,
+        hipLaunchKernelGGL(kvc_tail_values_kernel, dim3((unsigned)(batch * q_heads)), dim3(KVC_TAIL_WAVES * KVC_WAVE), 0, stream,
                            reinterpret_cast<const __half *>(v->d_tail_f16), scores, p.scores_stride, softmax_scale,
                            part + g * batch * q_heads * head_dim, ml + g * batch * q_heads * 2, v->tokens, v->tail_tokens,
                            (int)batch, (int)kv_heads, rep, (int)head_dim);
