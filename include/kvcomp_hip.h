@@ -71,7 +71,9 @@ int kvc_abi_version(void);
  *   "fused_rounded":         0 (default): the fused matvecs multiply q / p by (sym + min) * scale as it stands, in
  *                           fp32.  1: every such value is first rounded to fp16, as the reference's dequantizer
  *                           rounds it (models/cache/kvcomp_encode.py:146), so the result is the fp32 attention
- *                           over that fp16 cache; about half the speed.
+ *                           over that fp16 cache; about two thirds of the speed.
+ *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
+ *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile
  *                           pipeline; 0: on the simpler stand-alone kernels. */
 int kvc_set_option(const char *name, int value);

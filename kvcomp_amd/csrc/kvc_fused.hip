@@ -1516,16 +1516,31 @@ kvc_tail_values_kernel(const __half *__restrict__ tail, const float *__restrict_
 // together (indices past the end are clamped and weighted zero, so nothing branches around a load) -- and the
 // waves' sums are brought to the common maximum when they are merged: a 32k-token context is one round trip to
 // memory and one barrier.
+// With tail.n_v > 0 the same workgroup first handles the tokens that V keeps uncompressed (at most
+// KVC_FINISH_MAX_TAIL), as one more group: their scores (from the score matrix where K had them compressed, else
+// q . the fp16 row of K's tail), the group's maximum, the weights and the weighted sum of V's fp16 rows.
 constexpr int KVC_COMBINE_WAVES = 16;
+constexpr int KVC_FINISH_MAX_TAIL = KVC_COMBINE_WAVES * KVC_WAVE;
+struct KvcTailArgs {
+    const __half *k_tail, *v_tail, *q;    // [n_k, B, H, D], [n_v, B, H, D], [B, Hq, D]
+    const float *scores;                  // [B * Hq, scores_stride], filled for tokens below kc
+    int64_t scores_stride;
+    int64_t kc, vc;                       // tokens that K / V hold compressed (kc >= vc)
+    int n_k, n_v;                         // tokens in K's / V's fp16 tail (total - kc, total - vc)
+    float sm_scale;
+    int batch, kv_heads, rep;
+};
+
 template <int U>
 __global__ void __launch_bounds__(KVC_COMBINE_WAVES * KVC_WAVE)
 kvc_attention_combine_kernel(const float *__restrict__ part, const float *__restrict__ ml, int64_t groups,
-                             int64_t bhq_count, int D, float *__restrict__ out)
+                             int64_t bhq_count, int D, float *__restrict__ out, KvcTailArgs tail)
 {
     __shared__ float s_max[KVC_COMBINE_WAVES];
     __shared__ float s_num[KVC_COMBINE_WAVES][128];
     __shared__ float s_den[KVC_COMBINE_WAVES];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __shared__ float s_w[KVC_FINISH_MAX_TAIL];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t bhq = blockIdx.x;
     const int d0 = lane < D ? lane : 0, d1 = lane + 64 < D ? lane + 64 : 0;
     float M = -INFINITY, n0 = 0.f, n1 = 0.f, den = 0.f;   // this wave's running maximum and its sums relative to it
@@ -1559,6 +1574,63 @@ kvc_attention_combine_kernel(const float *__restrict__ part, const float *__rest
             n0 += f * p0[u];
             n1 += f * p1[u];
         }
+    }
+    if (tail.n_v > 0) {                                   // uniform over the workgroup
+        const int hq = (int)(bhq % (tail.kv_heads * tail.rep)), b = (int)(bhq / (tail.kv_heads * tail.rep));
+        const int h = hq / tail.rep;
+        const int from_k = (int)(tail.kc - tail.vc);      // tail tokens of V whose scores the K kernel wrote
+        // scaled scores of the tail tokens
+        if (tid < from_k) s_w[tid] = tail.scores[bhq * tail.scores_stride + tail.vc + tid] * tail.sm_scale;
+        {
+            const bool live = 2 * lane < D;
+            const int e = live ? 2 * lane : 0;
+            const __half2 qv = *reinterpret_cast<const __half2 *>(tail.q + bhq * D + e);
+            const float q0 = live ? __low2float(qv) : 0.f, q1 = live ? __high2float(qv) : 0.f;
+            const int64_t row = (int64_t)tail.batch * tail.kv_heads * D;
+            const __half *kp = tail.k_tail + ((int64_t)b * tail.kv_heads + h) * D + e;
+            for (int j = wave; j < tail.n_k; j += KVC_COMBINE_WAVES) {
+                const __half2 kv = *reinterpret_cast<const __half2 *>(kp + j * row);
+                const float dot = kvc_wave_sum_dpp(q0 * __low2float(kv) + q1 * __high2float(kv));
+                if (lane == 0) s_w[from_k + j] = dot * tail.sm_scale;
+            }
+        }
+        __syncthreads();
+        // the group's maximum, then every thread turns one score into a weight
+        const float sc = tid < tail.n_v ? s_w[tid] : -INFINITY;
+        float mt = kvc_wave_fmax_dpp(sc);
+        if (lane == 0) s_max[wave] = mt;
+        __syncthreads();
+        mt = s_max[0];
+#pragma unroll
+        for (int w = 1; w < KVC_COMBINE_WAVES; w++) mt = fmaxf(mt, s_max[w]);
+        const float wt = tid < tail.n_v ? __expf(sc - mt) : 0.f;
+        __syncthreads();                                  // every thread has read s_max and its score
+        s_w[tid] = wt;
+        const float lw = kvc_wave_sum_dpp(wt);            // this wave's share of the group's sum of weights
+        __syncthreads();
+        // weighted rows of V's tail: wave w takes tokens w, w + 16, ...; lane l channels l and l + 64
+        float a0 = 0.f, a1 = 0.f;
+        {
+            const int64_t row = (int64_t)tail.batch * tail.kv_heads * D;
+            const __half *vp = tail.v_tail + ((int64_t)b * tail.kv_heads + h) * D;
+            for (int j = wave; j < tail.n_v; j += KVC_COMBINE_WAVES) {
+                const float wj = s_w[j];
+                a0 += wj * __half2float(vp[j * row + d0]);
+                a1 += wj * __half2float(vp[j * row + d1]);
+            }
+        }
+        if (mt > M) {
+            const float f = __expf(M - mt);
+            n0 *= f;
+            n1 *= f;
+            den *= f;
+            M = mt;
+        }
+        const float f = __expf(mt - M);
+        den += f * lw;
+        n0 += f * a0;
+        n1 += f * a1;
+        __syncthreads();                                  // s_max is reused below
     }
     if (lane == 0) s_max[wave] = M;
     __syncthreads();
@@ -1645,7 +1717,27 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
                                k->max_tile_bytes, k->max_stream_bytes, k->max_code_bits, &ex))
             return rc;
     }
-    if (k->tail_tokens) {
+    // V's fp16 tail is handled by the merge kernel itself when it is short enough and K's compressed part reaches at
+    // least as far as V's (the V kernel then needs no score of K's tail); otherwise by two kernels of its own
+    KvcTailArgs tail = {};
+    const bool tail_in_merge = v->tail_tokens > 0 && v->tail_tokens <= KVC_FINISH_MAX_TAIL && k->tokens >= v->tokens &&
+                               kvc_option(KVC_OPT_ATTENTION_TAIL_IN_MERGE) != 0;
+    if (tail_in_merge) {
+        tail.k_tail = reinterpret_cast<const __half *>(k->d_tail_f16);
+        tail.v_tail = reinterpret_cast<const __half *>(v->d_tail_f16);
+        tail.q = reinterpret_cast<const __half *>(d_q_f16);
+        tail.scores = scores;
+        tail.scores_stride = p.scores_stride;
+        tail.kc = k->tokens;
+        tail.vc = v->tokens;
+        tail.n_k = (int)k->tail_tokens;
+        tail.n_v = (int)v->tail_tokens;
+        tail.sm_scale = softmax_scale;
+        tail.batch = (int)batch;
+        tail.kv_heads = (int)kv_heads;
+        tail.rep = rep;
+    }
+    if (k->tail_tokens && !tail_in_merge) {
         const int64_t items = k->tail_tokens * batch * kv_heads;
         hipLaunchKernelGGL(kvc_tail_scores_kernel, dim3((unsigned)((items + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG)), dim3(KVC_WG),
                            0, stream, reinterpret_cast<const __half *>(k->d_tail_f16), reinterpret_cast<const __half *>(d_q_f16),
@@ -1661,7 +1753,7 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
                                v->max_tile_bytes, v->max_stream_bytes, v->max_code_bits, &ex))
             return rc;
     }
-    if (v->tail_tokens) {
+    if (v->tail_tokens && !tail_in_merge) {
         const int64_t g = v->tokens / KVC_V_TOKENS;
         hipLaunchKernelGGL(kvc_tail_values_kernel, dim3((unsigned)(batch * q_heads)), dim3(KVC_TAIL_WAVES * KVC_WAVE), 0, stream,
                            reinterpret_cast<const __half *>(v->d_tail_f16), scores, p.scores_stride, softmax_scale,
@@ -1669,14 +1761,15 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
                            (int)batch, (int)kv_heads, rep, (int)head_dim);
     }
     // groups in flight per wave: what one pass over a wave's share needs, at most 16
+    const int64_t groups = tail_in_merge ? v->tokens / KVC_V_TOKENS : p.groups;
     const dim3 cgrid((unsigned)(batch * q_heads)), cblock(KVC_COMBINE_WAVES * KVC_WAVE);
-    const int64_t per_wave = (p.groups + KVC_COMBINE_WAVES - 1) / KVC_COMBINE_WAVES;
+    const int64_t per_wave = (groups + KVC_COMBINE_WAVES - 1) / KVC_COMBINE_WAVES;
     if (per_wave <= 4)
-        hipLaunchKernelGGL(kvc_attention_combine_kernel<4>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<4>, cgrid, cblock, 0, stream, part, ml, groups, batch * q_heads, (int)head_dim, d_out_f32, tail);
     else if (per_wave <= 8)
-        hipLaunchKernelGGL(kvc_attention_combine_kernel<8>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<8>, cgrid, cblock, 0, stream, part, ml, groups, batch * q_heads, (int)head_dim, d_out_f32, tail);
     else
-        hipLaunchKernelGGL(kvc_attention_combine_kernel<16>, cgrid, cblock, 0, stream, part, ml, p.groups, batch * q_heads, (int)head_dim, d_out_f32);
+        hipLaunchKernelGGL(kvc_attention_combine_kernel<16>, cgrid, cblock, 0, stream, part, ml, groups, batch * q_heads, (int)head_dim, d_out_f32, tail);
     KVC_HIP(hipGetLastError());
     return timer.finish();
 }
