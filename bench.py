@@ -173,9 +173,9 @@ def codec_rates(kctx, vctx, k, v, cfg):
 # what the same counter reads for the 256 MiB kvc_calibration_copy_kernel of the same run (FETCH_SIZE x2.0,
 # WRITE_SIZE x1.0).  Source: profiles/fused_decode_attention_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
-    "cfg2": {"kvc_fused_kernel<1, 0>": int((4084.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2740.9 * 2.0 + 528.0) * 1024)},
-    "cfg3": {"kvc_fused_kernel<4, 0>": int((31975.8 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, 3>": int((26482.6 * 2.0 + 16640.0) * 1024)},
-    "cfg5": {"kvc_fused_kernel<1, 0>": int((102580.6 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((45756.6 * 2.0 + 12743.3) * 1024)},
+    "cfg2": {"kvc_fused_kernel<1, 0>": int((4087.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2758.4 * 2.0 + 528.0) * 1024)},
+    "cfg3": {"kvc_fused_kernel<4, 0>": int((31971.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, 3>": int((26478.8 * 2.0 + 16640.0) * 1024)},
+    "cfg5": {"kvc_fused_kernel<1, 0>": int((102552.1 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((45746.0 * 2.0 + 12743.3) * 1024)},
 }
 
 
