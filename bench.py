@@ -260,6 +260,7 @@ def main():
     ap.add_argument("--eb-k", type=float, default=None, help="override the K error bound of the workload (cfg5 sweeps 0.05 / 0.1 / 0.2)")
     ap.add_argument("--no-rounded", action="store_true",
                     help="skip the extra pass in rounded mode (keeps a kernel trace of this run to one variant per kernel)")
+    ap.add_argument("--no-graph", action="store_true", help="skip the replay of the step as a captured HIP graph")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 256 MiB device copy (kvc_calibration_copy_kernel), the yardstick "
                          "for FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -356,6 +357,30 @@ def main():
             _lib.set_option("fused_rounded", was)
         log("[bench] rounded mode: step %.3f ms" % rounded_ms)
 
+    # the same step captured once in a HIP graph and replayed (what a serving loop does with a launch-bound step:
+    # the library call allocates nothing and waits for nothing, so it can be recorded as it is)
+    graph_ms = None
+    if not args.no_graph:
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            attn.attend(q, out=out)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=side):
+                attn.attend(q, out=out)
+        torch.cuda.synchronize()
+        eager = attn.attend(q).clone()
+        for _ in range(args.warmup):
+            graph.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            graph.replay()
+        torch.cuda.synchronize()
+        graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        assert torch.equal(out, eager), "graph replay differs from the eager call"
+        log("[bench] one step as a HIP graph, replayed: %.3f ms" % graph_ms)
+
     # template arguments: query heads per KV head, then 0 = K tile, 3 / 4 = V tile with the softmax on the fly
     # (4: head_dim is not a multiple of 64, tiles may straddle two heads)
     v_kind = 3 if D % 64 == 0 else 4
@@ -378,6 +403,7 @@ def main():
                                         "arithmetic": "q . ((sym + min) * scale) with the dequantized value kept in fp32 (within 1e-4 of "
                                                       "fp64 attention over that dequantization); rounded_mode rounds it to fp16 first like "
                                                       "the reference's dequantizer (within 1e-3 of fp32 attention over the fp16 cache)",
+                                        "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
                                         "rounded_mode": None if rounded_ms is None else
                                         {"ms_per_step": round(rounded_ms, 4), "GBs": round((kb + vb) / (rounded_ms * 1e-3) / 1e9, 1)},
                                         "symbols_per_s": {"fused_k": round(numel / k_ms * 1e3), "fused_v": round(numel / v_ms * 1e3)},

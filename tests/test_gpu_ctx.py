@@ -303,3 +303,39 @@ def test_one_kernel_get_equals_decode_then_dequant(is_k, mode, B, H, D):
     o = O.quant(S.np16(S.blocked(x, ctx.block_size)), mask, 0.1)
     deq = O.dequant(o[3], o[4], o[2], mask).reshape(T, B, H, D)
     assert np.array_equal(one.cpu().numpy().view(np.uint16), deq.view(np.uint16))
+
+
+def test_attention_call_can_be_captured_in_a_graph():
+    """kvc_attention_decode allocates nothing and waits for nothing, so a serving loop can record it in a HIP graph.
+    The graph is replayed several times with eager work and synchronisations of the program's own in between, for
+    queries that change between replays (the graph reads q and writes out in place), with and without fp16 tails;
+    every replay must equal the eager call bit for bit."""
+    from kvcomp_amd.attention import CompressedAttention
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    B, H, Hq, D = 2, 2, 8, 128
+    for T in (512, 512 + 37):
+        k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+        kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+        kctx.store(k)
+        vctx.store(v)
+        attn = CompressedAttention(kctx, vctx)
+        q = S.synth_q(B, Hq, D).to(DEV)
+        out = torch.empty(B, Hq, D, dtype=torch.float32, device=DEV)
+        attn.attend(q, out=out)                                   # builds the tables and the workspace
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                attn.attend(q, out=out)
+        torch.cuda.synchronize()
+        g = torch.Generator(device=DEV).manual_seed(4)
+        for i in range(4):
+            q.copy_(torch.randn(B, Hq, D, generator=g, device=DEV).to(torch.float16))
+            eager = attn.attend(q).clone()                        # eager work between the replays
+            torch.cuda.synchronize()
+            out.fill_(float("nan"))
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), (T, i)
