@@ -14,6 +14,17 @@ bring their own attention loop.
     KVCompCacheConfigStatic.config = KVCompCacheConfig(...)          # as for the reference
     cache = KVCompHFCache(num_layers)
     out = model(input_ids, past_key_values=cache, use_cache=True)
+
+A model can also be told to attend on the compressed form by itself: `register_kvcomp_attention()` adds the
+attention implementation "kvcomp" to transformers' registry, and a cache built with `attend_compressed=True` then
+stops decompressing the history on single-token steps -- `update` stores the token and hands the attention
+function a tagged placeholder, the function runs `kvc_attention_decode` over the layer's streams.  Prompts (more
+than one query token) still get the dense (K, V) and the stock scaled-dot-product attention.
+
+    register_kvcomp_attention()
+    model.set_attn_implementation("kvcomp")
+    cache = KVCompHFCache(attend_compressed=True)
+    model.generate(input_ids, past_key_values=cache, ...)            # unpadded batches, greedy or sampling
 """
 from typing import Optional, Tuple
 
@@ -35,6 +46,7 @@ class KVCompLayer(CacheLayerMixin):
         self.k_ctx: Optional[KVCompCtx] = None
         self.v_ctx: Optional[KVCompCtx] = None
         self._attention: Optional[CompressedAttention] = None
+        self.attend_compressed = False      # single-token steps: no dense history, the attention function attends here
 
     def lazy_initialization(self, key_states: torch.Tensor, value_states: torch.Tensor) -> None:
         cfg = KVCompCacheConfigStatic.config
@@ -54,6 +66,11 @@ class KVCompLayer(CacheLayerMixin):
             self.lazy_initialization(key_states, value_states)
         self.k_ctx.store(key_states.permute(2, 0, 1, 3).contiguous(), want_symbols=False)
         self.v_ctx.store(value_states.permute(2, 0, 1, 3).contiguous(), want_symbols=False)
+        if self.attend_compressed and key_states.shape[2] == 1:
+            # kvcomp_attention_forward recognises the tag and attends on the compressed streams of this layer
+            key_states._kvcomp_layer = self
+            self.keys = self.values = None
+            return key_states, value_states
         self.keys = self.k_ctx.get()[0].permute(1, 2, 0, 3)
         self.values = self.v_ctx.get()[0].permute(1, 2, 0, 3)
         return self.keys, self.values
@@ -109,11 +126,21 @@ class KVCompLayer(CacheLayerMixin):
 class KVCompHFCache(Cache):
     """`Cache` of KVCompLayer objects; one per decoder layer, or grown on demand when `num_layers` is None."""
 
-    def __init__(self, num_layers: Optional[int] = None):
+    def __init__(self, num_layers: Optional[int] = None, attend_compressed: bool = False):
+        self.attend_compressed = attend_compressed
         if num_layers is None:
             super().__init__(layer_class_to_replicate=KVCompLayer)
         else:
             super().__init__(layers=[KVCompLayer() for _ in range(num_layers)])
+        for layer in self.layers:
+            layer.attend_compressed = attend_compressed
+
+    def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int, *args, **kwargs):
+        while self.attend_compressed and len(self.layers) <= layer_idx:          # layers grown on demand
+            self.layers.append(KVCompLayer())
+        if self.attend_compressed:
+            self.layers[layer_idx].attend_compressed = True
+        return super().update(key_states, value_states, layer_idx, *args, **kwargs)
 
     def attend(self, layer_idx: int, query: torch.Tensor, softmax_scale: Optional[float] = None) -> torch.Tensor:
         return self.layers[layer_idx].attend(query, softmax_scale)
@@ -130,3 +157,26 @@ class KVCompHFCache(Cache):
                 dense += 2 * 2 * c.ctx_len * c.batch_size * c.head_num * c.head_dim
         held = self.compressed_bytes()
         return dense / held if held else 1.0
+
+
+def kvcomp_attention_forward(module, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attention_mask,
+                             dropout: float = 0.0, scaling: Optional[float] = None, **kwargs):
+    """Attention implementation "kvcomp" for transformers' registry.  A single query token whose key carries the tag
+    of a KVCompLayer (see KVCompLayer.update) is answered by decode attention over that layer's compressed streams:
+    query [B, H_q, 1, D] -> ([B, 1, H_q, D], None).  Everything else goes to the stock scaled-dot-product attention.
+    The compressed path attends over every stored token of every sequence (no padding mask)."""
+    layer = getattr(key, "_kvcomp_layer", None)
+    if layer is None or query.shape[2] != 1:
+        from transformers.integrations.sdpa_attention import sdpa_attention_forward
+        return sdpa_attention_forward(module, query, key, value, attention_mask, dropout=dropout, scaling=scaling, **kwargs)
+    out = layer.attend(query[:, :, 0, :].contiguous(), scaling)                  # fp32 [B, H_q, D]
+    return out.to(query.dtype).unsqueeze(1), None
+
+
+def register_kvcomp_attention(name: str = "kvcomp") -> str:
+    """Make `name` selectable as a model's attention implementation (masks as for "sdpa").  Idempotent."""
+    from transformers import AttentionInterface
+    from transformers.masking_utils import AttentionMaskInterface, sdpa_mask
+    AttentionInterface.register(name, kvcomp_attention_forward)
+    AttentionMaskInterface.register(name, sdpa_mask)
+    return name

@@ -99,3 +99,54 @@ def test_generate_with_the_compressed_cache():
     out = model.generate(ids, past_key_values=cache, max_new_tokens=80, do_sample=False, use_cache=True, pad_token_id=0)
     assert out.shape == (1, 280) and cache.get_seq_length() == 279
     assert cache.layers[0].k_ctx.compressed_ctx_len == 256 and cache.layers[0].v_ctx.compressed_ctx_len == 256   # (279 - 279 % bs) / bs + 1 - recent / bs blocks
+
+
+def test_model_attends_on_the_compressed_cache_through_the_attention_registry():
+    """With the attention implementation "kvcomp" and a cache built with attend_compressed=True, single-token steps
+    never decompress the history: update() stores the token and the registered attention function runs the fused
+    decode attention of the layer.  Logits must agree with the same model reading the dense (K, V) that the
+    compressed cache hands out otherwise (the two differ only by fp16 rounding of the dequantized cache and of
+    the stock attention's arithmetic); prompts still take the dense path."""
+    from kvcomp_amd import hf_adapter as HA
+    _config(0.1, 0.2)
+    model = _tiny_llama()
+    name = HA.register_kvcomp_attention()
+    g = torch.Generator().manual_seed(9)
+    B = 2
+    ids = torch.randint(0, 256, (B, 300), generator=g).to(DEV)
+    dense_like, lazy = HA.KVCompHFCache(), HA.KVCompHFCache(attend_compressed=True)
+    calls = {"n": 0}
+    real_attend = HA.KVCompLayer.attend
+
+    def counting_attend(self, *a, **k):
+        calls["n"] += 1
+        return real_attend(self, *a, **k)
+
+    HA.KVCompLayer.attend = counting_attend
+    try:
+        sims, diffs = [], []
+        with torch.no_grad():
+            model.set_attn_implementation("sdpa")
+            model(ids[:, :256], past_key_values=dense_like, use_cache=True)
+            model.set_attn_implementation(name)
+            model(ids[:, :256], past_key_values=lazy, use_cache=True)          # a prompt: dense path, no attend() call
+            assert calls["n"] == 0
+            for t in range(256, 300):
+                model.set_attn_implementation("sdpa")
+                a = model(ids[:, t:t + 1], past_key_values=dense_like, use_cache=True).logits[:, -1].float()
+                model.set_attn_implementation(name)
+                b = model(ids[:, t:t + 1], past_key_values=lazy, use_cache=True).logits[:, -1].float()
+                sims.append(float(torch.nn.functional.cosine_similarity(a, b, dim=-1).min()))
+                diffs.append(float((a - b).abs().max() / a.abs().max()))
+        n_layers = model.config.num_hidden_layers
+        assert calls["n"] == 44 * n_layers                                      # every decode step of every layer
+        assert lazy.get_seq_length() == dense_like.get_seq_length() == 300
+        assert all(layer.keys is None for layer in lazy.layers)                  # no dense history was produced
+        assert min(sims) > 0.999 and max(diffs) < 2e-2, (min(sims), max(diffs))
+        # and generation runs end to end
+        model.set_attn_implementation(name)
+        cache = HA.KVCompHFCache(attend_compressed=True)
+        out = model.generate(ids[:, :200], past_key_values=cache, max_new_tokens=40, do_sample=False, use_cache=True)
+        assert out.shape == (B, 240) and cache.get_seq_length() == 239
+    finally:
+        HA.KVCompLayer.attend = real_attend
