@@ -250,6 +250,77 @@ def run_decode_loop(args):
     print(json.dumps(result), flush=True)
 
 
+def run_model_decode(args):
+    """cfg4 as BASELINE.json words it: the Llama-2-7B architecture with random-init fp16 weights (stock `transformers`
+    modelling code), a compressed KV cache in every layer, batch 8, a 4096-token random prompt and greedy generation;
+    single-token steps attend on the compressed form through the "kvcomp" attention implementation.  Tokens are random,
+    so the text means nothing; the arithmetic and the memory traffic are those of the real model."""
+    import torch
+    from transformers import LlamaConfig, LlamaForCausalLM
+    from kvcomp_amd import hf_adapter as HA
+    from kvcomp_amd.ctx import KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
+    cfg = WORKLOADS["cfg4"]
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    L = args.model_layers
+    B, H, D, T = cfg["B"], cfg["H"], cfg["D"], cfg["T"]
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("cfg4", QuantMode.ChannelQuant, QuantMode.TokenQuant,
+                                                       64, 128, 64, 128, cfg["eb_k"], cfg["eb_v"])
+    log("[bench] Llama-2-7B architecture, %d layers, random fp16 weights, batch %d, %d-token prompt, %d generated tokens"
+        % (L, B, T, args.new_tokens))
+    mcfg = LlamaConfig(vocab_size=32000, hidden_size=H * D, intermediate_size=11008, num_hidden_layers=L,
+                       num_attention_heads=H, num_key_value_heads=H, max_position_embeddings=T + args.new_tokens + 64,
+                       attn_implementation="sdpa")
+    torch.manual_seed(1240)
+    old_dtype = torch.get_default_dtype()
+    torch.set_default_dtype(torch.float16)
+    try:
+        with torch.device(dev):
+            model = LlamaForCausalLM(mcfg).eval()
+    finally:
+        torch.set_default_dtype(old_dtype)
+    g = torch.Generator().manual_seed(1239)
+    ids = torch.randint(0, 32000, (B, T), generator=g).to(dev)
+    if args.dense_cache:                     # comparison run: transformers' own fp16 cache and attention
+        from transformers import DynamicCache
+        cache = DynamicCache()
+    else:
+        model.set_attn_implementation(HA.register_kvcomp_attention())
+        cache = HA.KVCompHFCache(attend_compressed=True)
+    with torch.no_grad():
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        logits = model(ids, past_key_values=cache, use_cache=True, logits_to_keep=1).logits
+        nxt = logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        t_prefill = time.perf_counter() - t0
+        for _ in range(args.warmup):
+            nxt = model(nxt, past_key_values=cache, use_cache=True).logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.new_tokens):
+            nxt = model(nxt, past_key_values=cache, use_cache=True).logits[:, -1].argmax(-1, keepdim=True)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    result = {
+        "metric": "decode tokens/s, Llama-2-7B architecture (random weights) with a compressed KV cache in every layer",
+        "value": round(B * args.new_tokens / dt, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.new_tokens,
+        "warmup": args.warmup, "ms_per_step": round(dt / args.new_tokens * 1e3, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "fp16 model, u8 symbols, fp32 accumulate in attention",
+        "data": "synthetic",
+        "config": {"workload": "cfg4 with the model: %d layers, batch %d, %d-token prompt, greedy decoding" % (L, B, T),
+                   "context_at_end": cache.get_seq_length(),
+                   "compression_ratio_whole_cache": None if args.dense_cache else round(cache.compression_ratio(), 3),
+                   "cache_bytes_held": (2 * 2 * L * cache.get_seq_length() * B * H * D if args.dense_cache
+                                        else cache.compressed_bytes()),
+                   "prefill_s": round(t_prefill, 3),
+                   "attention": ("transformers DynamicCache (dense fp16) and stock SDPA: the comparison run" if args.dense_cache else
+                                 "single-token steps: kvc_attention_decode on the compressed streams; prompt: stock SDPA")},
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -261,6 +332,12 @@ def main():
     ap.add_argument("--no-rounded", action="store_true",
                     help="skip the extra pass in rounded mode (keeps a kernel trace of this run to one variant per kernel)")
     ap.add_argument("--no-graph", action="store_true", help="skip the replay of the step as a captured HIP graph")
+    ap.add_argument("--model-layers", type=int, default=0,
+                    help="cfg4 only: run the Llama-2-7B architecture itself (random weights) with this many layers (32 = "
+                         "the whole model) instead of the cache-and-attention loop")
+    ap.add_argument("--dense-cache", action="store_true",
+                    help="cfg4 with --model-layers: use transformers' dense fp16 cache and attention instead (comparison run)")
+    ap.add_argument("--new-tokens", type=int, default=256, help="cfg4 with --model-layers: tokens generated after the prompt")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch one plain 256 MiB device copy (kvc_calibration_copy_kernel), the yardstick "
                          "for FETCH_SIZE / WRITE_SIZE when this command runs under rocprofv3 --pmc")
@@ -275,7 +352,7 @@ def main():
     from kvcomp_amd import attention as A
 
     if args.workload == "cfg4":
-        return run_decode_loop(args)
+        return run_model_decode(args) if args.model_layers > 0 else run_decode_loop(args)
     cfg = dict(WORKLOADS[args.workload])
     if args.eb_k is not None:
         cfg["desc"] = cfg["desc"].replace("eb K %g" % cfg["eb_k"], "eb K %g" % args.eb_k)
