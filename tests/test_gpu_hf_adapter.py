@@ -150,3 +150,46 @@ def test_model_attends_on_the_compressed_cache_through_the_attention_registry():
         assert out.shape == (B, 240) and cache.get_seq_length() == 239
     finally:
         HA.KVCompLayer.attend = real_attend
+
+
+def _tiny(family):
+    import transformers as tf
+    torch.manual_seed(0)
+    if family == "mistral":                                   # grouped-query attention, 4 query heads per KV head
+        cfg = tf.MistralConfig(vocab_size=256, hidden_size=512, intermediate_size=512, num_hidden_layers=2, num_attention_heads=8,
+                               num_key_value_heads=2, head_dim=64, max_position_embeddings=1024, sliding_window=None,
+                               attn_implementation="sdpa")
+        return tf.MistralForCausalLM(cfg).to(DEV).to(torch.float16).eval()
+    if family == "phi3":                                      # head_dim 96, fused qkv projection
+        cfg = tf.Phi3Config(vocab_size=256, hidden_size=384, intermediate_size=512, num_hidden_layers=2, num_attention_heads=4,
+                            num_key_value_heads=4, max_position_embeddings=1024, original_max_position_embeddings=1024,
+                            sliding_window=None, pad_token_id=0, attn_implementation="sdpa")
+        return tf.Phi3ForCausalLM(cfg).to(DEV).to(torch.float16).eval()
+    raise ValueError(family)
+
+
+@pytest.mark.parametrize("family", ["mistral", "phi3"])
+def test_other_architectures_attend_on_the_compressed_cache(family):
+    """The model families the reference forks (models/mistral.py, models/phi3.py), as stock transformers code: grouped
+    queries (4 per KV head) and head_dim 96 go through the same registered attention function."""
+    from kvcomp_amd import hf_adapter as HA
+    _config(0.1, 0.2)
+    model = _tiny(family)
+    name = HA.register_kvcomp_attention()
+    g = torch.Generator().manual_seed(19)
+    ids = torch.randint(1, 256, (2, 290), generator=g).to(DEV)
+    dense_like, lazy = HA.KVCompHFCache(), HA.KVCompHFCache(attend_compressed=True)
+    sims = []
+    with torch.no_grad():
+        model.set_attn_implementation("sdpa")
+        model(ids[:, :256], past_key_values=dense_like, use_cache=True)
+        model.set_attn_implementation(name)
+        model(ids[:, :256], past_key_values=lazy, use_cache=True)
+        for t in range(256, 290):
+            model.set_attn_implementation("sdpa")
+            a = model(ids[:, t:t + 1], past_key_values=dense_like, use_cache=True).logits[:, -1].float()
+            model.set_attn_implementation(name)
+            b = model(ids[:, t:t + 1], past_key_values=lazy, use_cache=True).logits[:, -1].float()
+            sims.append(float(torch.nn.functional.cosine_similarity(a, b, dim=-1).min()))
+    assert all(layer.keys is None for layer in lazy.layers) and lazy.get_seq_length() == 290
+    assert min(sims) > 0.999, min(sims)
