@@ -1,32 +1,38 @@
 // kvc_fused.hip -- Huffman decode fused with the two matvecs of decode attention: decoded symbols go
 // from the LDS lookup straight into an fp32 FMA and never reach HBM.
 //
-//   kvc_fused_kernel<REP, true>   <- huffman_decode_and_mat_vec_mul   (kvcomp_cuda_extension/src/kernels.cu:721-776)
-//   kvc_fused_kernel<REP, false>  <- v_huffman_decode_and_mat_vec_mul (kernels.cu:778-861)
+//   kvc_fused_kernel<REP, 0>      <- huffman_decode_and_mat_vec_mul   (kvcomp_cuda_extension/src/kernels.cu:721-776)
+//   kvc_fused_kernel<REP, 1 .. 4> <- v_huffman_decode_and_mat_vec_mul (kernels.cu:778-861); 3 / 4 form the softmax
+//                                    weights of each 128-token group from raw scores on the fly
+//   kvc_expand_kernel<KIND, DEQ>  <- huffman_decode / v_huffman_decode (kernels.cu:602-719) on the same pipeline
+//   kvc_attention_decode          one call per layer: fused K, fused V, merge (+ the fp16 tails)
 //
 // One wave64 per tile, lane t owns stream t (K: a token, V: a channel), exactly the reference's work split.
-// Every lane decodes one symbol per step, so step i means "channel i" (K) or "token i of the 128-token
-// group" (V) for the whole wave and the other FMA operand is wave-uniform:
+// Every lane decodes one symbol (or exactly two, with the pair table) per step, so step i means "channel i" (K)
+// or "token i of the 128-token group" (V) for the whole wave and the other FMA operand is wave-uniform:
 //   K: score  = sum_i (sym_i + min_i) scale_i q_i = sum_i sym_i q'_i + sum_i min_i q'_i,  q'_i = scale_i q_i
 //   V: out_d  = sum_t (sym_t + min_t) scale_t p_t = sum_t sym_t w_t  + sum_t min_t w_t,   w_t  = scale_t p_t
-// q' / w are computed once per tile into two VGPRs per query head (lane l holds elements l and l + 64) and
-// reach the FMA through v_readlane.  REP query heads share one KV head (grouped-query attention): the tile
-// is decoded once and feeds REP accumulators.
+// q' / w are computed once per tile into an operand table in LDS; lane l reads element 4k + (l & 3) of every
+// block of four and the FMA picks its operand from the right lane of the quad (a DPP modifier, no instruction).
+// REP query heads share one KV head (grouped-query attention): the tile is decoded once and feeds REP accumulators.
 //
-// Inner loop (the "fast" path, codes no longer than the table index).  The payload is staged in LDS with
-// every 32-bit word bit-reversed, so stream bit k is bit (k & 31) of word k >> 5 and a window is a plain
-// right funnel shift:
+// Pipeline per wave: everything a tile needs from global memory is fetched into registers one tile ahead;
+// staging converts the payload to least-significant-bit-first words in LDS (optionally with two spare words per
+// 32, which spreads lanes that would otherwise share a bank), builds the operand table and reduces the constant
+// term with DPP steps.
+//
+// Inner loop (the "fast" path, codes no longer than the table index):
 //   window  32 stream bits, least significant first, held two bits up: the next `lbits` bits sit at bits
 //           [lbits+1 : 2], so masking gives the byte offset of the table entry directly
 //   entry   fp32 bit pattern of the symbol with the code length in its lowest mantissa byte: it is the FMA
 //           operand as it stands, and as a shift count it rotates the window right by len (v_alignbit)
-//   refill  every 4 (or 8) symbols the window is re-read from the staged payload at the lane's bit position
-//           (one ds_read2_b32 + one v_alignbit); the entries are summed, and the low byte of the sum is the
-//           number of bits consumed
-// A 32-bit window always suffices for 8 symbols of <= 4 bits or 4 symbols of <= 8 bits (two of the 32 bits
-// are the look-behind pair, hence 30 usable).  With longer codes 4 symbols can, very rarely, need more:
-// lanes note the largest consumption they saw, and if any lane went over, the wave decodes that tile again
-// on the slow path.
+//   refill  64 stream bits (three words, two funnel shifts): G symbols from the low half, the window re-formed
+//           from the register pair at the bits consumed, G more; G = what a 30-bit window is sure to hold
+//           (30 / longest code, at most 8); the entries are summed and the low byte of the sum is the number
+//           of bits consumed
+//   pairs   with codes of at most 4 bits a table of 8-byte entries yields two symbols per look-up
+// Codebooks whose average code is short may use a larger G than is safe; lanes then note the largest
+// consumption they saw, and if any lane went over, the wave decodes that tile again on the slow path.
 //
 // Slow path (codebooks with codes longer than the table index, tiles larger than the staging area, or
 // the rare overflow above): one symbol per refill, generic table read from global memory, payload read
