@@ -2,15 +2,17 @@
 //
 // Replaces huffman_encode / v_huffman_encode and their launchers
 // (kvcomp_cuda_extension/src/kernels.cu:181-235, 419-596, 919-1011).  One wave64 per tile, lane t owns
-// vector t, as one 64-thread block does in the reference.  Three launches:
+// vector t, as one 64-thread block does in the reference.  The launches:
 //
 //   count  every lane adds up the code lengths of its vector; a wave prefix scan turns the 64 byte
 //          counts into thread_infos and the tile's byte_num           (kernels.cu:448-465, 472-478)
-//   scan   one workgroup turns the byte_nums into tile offsets, in tile order (the reference claims
+//   scan   payload bytes per 1024 tiles, then every workgroup turns the byte_nums of its own 1024 tiles
+//          into offsets, in tile order, without waiting for another workgroup (the reference claims
 //          offsets with a global atomic in arrival order, kernels.cu:474, which makes its stream
 //          layout differ from run to run)
 //   emit   every lane packs its codes MSB-first straight at its final position inside an LDS image
-//          of the tile payload (words it shares with a neighbour lane are merged with LDS atomic OR),
+//          of the tile payload (words it shares with a neighbour lane are merged with LDS atomic OR;
+//          four codes of at most 8 bits are joined before they enter the lane's 64-bit accumulator),
 //          and the wave copies the image out with aligned dword stores        (kernels.cu:181-235, 483-488)
 //
 // The symbols are read twice (1 B/symbol each) instead of once, which buys deterministic output
