@@ -280,6 +280,21 @@ int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_compressed_desc
                          int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
                          float *elapsed_ms, float *fused_kernel_ms, void *stream);
 
+/* ---- decode attention without any allocation (no counterpart in the reference; for callers that cannot
+ * allocate device memory: code under HIP graph capture, serving loops with a fixed memory plan, harnesses that
+ * forbid hipMalloc) --------------------------------------------------------------------------------------------
+ * kvc_attention_decode with the workspace kept in a device array of the library itself
+ * (KVC_ATTENTION_STATIC_SCRATCH_BYTES per GPU the library runs on, held until the process ends) instead of a
+ * caller's buffer; same arguments otherwise, no timing outputs, same results bit for bit.  Shapes whose workspace
+ * (kvc_attention_workspace_bytes) exceeds the array are rejected with an error.  The call itself allocates
+ * nothing and frees nothing.  The first call on a device looks the array's address up (make that call outside
+ * graph capture).  Calls that overlap in time on one device share the array and race: keep them on one stream
+ * or order them. */
+#define KVC_ATTENTION_STATIC_SCRATCH_BYTES (40 * 1024 * 1024)
+int kvc_attention_decode_static(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                                float softmax_scale, float *d_out_f32, int64_t batch, int64_t kv_heads,
+                                int64_t q_heads, int64_t head_dim, void *stream);
+
 /* ---- dense baseline: k_mat_vec_mul_cuda_export (kernels.cu:1182-1273) ------------------------------
  * d_k fp16 [tokens, batch, heads, head_dim], d_q fp16 [batch, heads, head_dim],
  * d_out fp16 [tokens, batch, heads].  (The reference requires batch == 1 and head_dim == 128.) */

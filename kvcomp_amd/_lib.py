@@ -65,6 +65,8 @@ _SIGNATURES = {
     "kvc_attention_workspace_bytes": [_i64, _i64, _i64, _i64, _i64],
     "kvc_attention_decode": [C.POINTER(CompressedDesc), C.POINTER(CompressedDesc), _vp, C.c_float, _vp, _i64, _vp,
                              _i64, _i64, _i64, _i64, _f32p, _f32p, _vp],
+    "kvc_attention_decode_static": [C.POINTER(CompressedDesc), C.POINTER(CompressedDesc), _vp, C.c_float, _vp,
+                                    _i64, _i64, _i64, _i64, _vp],
     "kvc_dequant": [_vp, _vp, _vp, _i64, _i64, _i64, _i64, _i64, _int, _vp, _vp],
 }
 _RESTYPES = {"kvc_quant_groups": _i64, "kvc_lut_bytes": _i64, "kvc_codebook_tree_capacity": _i64, "kvc_attention_workspace_bytes": _i64,

@@ -39,6 +39,7 @@
 // from LDS or -- for an oversized tile -- from global memory.
 #include "kvc_tile.h"
 
+#include <mutex>
 #include <type_traits>
 
 struct KvcFusedArgs {
@@ -1688,10 +1689,10 @@ extern "C" int64_t kvc_attention_workspace_bytes(int64_t total_tokens, int64_t v
     return kvc_attention_plan(total_tokens, v_compressed_tokens, batch, q_heads, head_dim).bytes;
 }
 
-extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
-                                    float softmax_scale, void *d_workspace, int64_t workspace_bytes, float *d_out_f32,
-                                    int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
-                                    float *elapsed_ms, float *fused_kernel_ms, void *stream_)
+static int kvc_attention_run(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                             float softmax_scale, void *d_workspace, int64_t workspace_bytes, float *d_out_f32,
+                             int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                             float *elapsed_ms, float *fused_kernel_ms, void *stream_)
 {
     hipStream_t stream = (hipStream_t)stream_;
     if (fused_kernel_ms) fused_kernel_ms[0] = fused_kernel_ms[1] = 0.f;
@@ -1778,4 +1779,63 @@ extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_comp
         hipLaunchKernelGGL(kvc_attention_combine_kernel<16>, cgrid, cblock, 0, stream, part, ml, groups, batch * q_heads, (int)head_dim, d_out_f32, tail);
     KVC_HIP(hipGetLastError());
     return timer.finish();
+}
+
+extern "C" int kvc_attention_decode(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                                    float softmax_scale, void *d_workspace, int64_t workspace_bytes, float *d_out_f32,
+                                    int64_t batch, int64_t kv_heads, int64_t q_heads, int64_t head_dim,
+                                    float *elapsed_ms, float *fused_kernel_ms, void *stream_)
+{
+    return kvc_attention_run(k, v, d_q_f16, softmax_scale, d_workspace, workspace_bytes, d_out_f32, batch, kv_heads,
+                             q_heads, head_dim, elapsed_ms, fused_kernel_ms, stream_);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The same operator for callers that may not allocate (code under HIP graph capture, serving loops with a
+// fixed memory plan): the workspace (scores, per-group partials and their (max, sum) pairs) lives in a
+// device array of this library instead of a caller's buffer.  Every device holds its own copy of the
+// array at its own address; the address is looked up once per device, on the first call there, and only
+// that pointer -- never the array's name, which in host code is a stand-in and not a device address --
+// is handed to the kernels.  Nothing in the workspace has to start at zero: every word the kernels read
+// is written earlier in the same call (scores by the K kernel, partials and (max, sum) by the V kernel),
+// at offsets that depend on this call's shape alone, so what an earlier, larger call left behind is
+// never read.  Calls that overlap in time on one device share the array and race.
+// ---------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[KVC_ATTENTION_STATIC_SCRATCH_BYTES];
+constexpr int KVC_SCRATCH_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[KVC_SCRATCH_MAX_DEVICES] = {};
+
+static int kvc_static_scratch(void **ptr)
+{
+    int dev = 0;
+    KVC_HIP(hipGetDevice(&dev));
+    KVC_REQUIRE(dev >= 0 && dev < KVC_SCRATCH_MAX_DEVICES, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        KVC_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        KVC_REQUIRE(p != nullptr && ((uintptr_t)p & 255) == 0, "the static workspace has no usable device address");
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int kvc_attention_decode_static(const kvc_compressed_desc *k, const kvc_compressed_desc *v, const void *d_q_f16,
+                                           float softmax_scale, float *d_out_f32, int64_t batch, int64_t kv_heads,
+                                           int64_t q_heads, int64_t head_dim, void *stream_)
+{
+    KVC_REQUIRE(k != nullptr && v != nullptr, "NULL argument");
+    KVC_REQUIRE(batch > 0 && q_heads > 0 && head_dim > 0, "batch, q_heads and head_dim must be positive");
+    const int64_t total = k->tokens + k->tail_tokens;
+    KVC_REQUIRE(total > 0 && v->tokens >= 0, "the cache is empty");
+    const int64_t need = kvc_attention_plan(total, v->tokens, batch, q_heads, head_dim).bytes;
+    KVC_REQUIRE(need <= (int64_t)KVC_ATTENTION_STATIC_SCRATCH_BYTES,
+                "this shape needs a workspace of %lld bytes, the static one holds %lld: use kvc_attention_decode",
+                (long long)need, (long long)KVC_ATTENTION_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    if (int rc = kvc_static_scratch(&ws)) return rc;
+    return kvc_attention_run(k, v, d_q_f16, softmax_scale, ws, (int64_t)KVC_ATTENTION_STATIC_SCRATCH_BYTES, d_out_f32, batch,
+                             kv_heads, q_heads, head_dim, nullptr, nullptr, stream_);
 }
