@@ -68,10 +68,14 @@ int kvc_abi_version(void);
  *   "fused_tiles_per_wave":  0 (default) chosen per call; n > 0: consecutive tiles one wave works through.
  *   "fused_pair_bits":       widest index of the two-symbols-per-look-up table (default 8; 0 = one symbol per look-up).
  *   "fused_double_window":   1 (default): 64 stream bits per refill in the one-symbol loops; 0: 32.
- *   "fused_rounded":         0 (default): the fused matvecs multiply q / p by (sym + min) * scale as it stands, in
- *                           fp32.  1: every such value is first rounded to fp16, as the reference's dequantizer
- *                           rounds it (models/cache/kvcomp_encode.py:146), so the result is the fp32 attention
- *                           over that fp16 cache; about two thirds of the speed.
+ *   "fused_rounded":         1 (default): the fused matvecs round every (sym + min) * scale to fp16 before it meets
+ *                           q / p, as the reference's dequantizer rounds it (models/cache/kvcomp_encode.py:146), so the
+ *                           result is the fp32 attention over that fp16 cache (within 1e-3).  0: the product is used
+ *                           as it stands, in fp32 (closer to exact arithmetic over the unrounded dequantization, and
+ *                           further from the reference's cache: a few 1e-3 on outlier-heavy data).
+ *   "fused_mfma":           -1 (default): the multiply-accumulate of the fused matvecs runs on the matrix cores
+ *                           (v_mfma_f32_4x4x4_16b_f16) where that is the faster kernel (rounded mode, codes of at most
+ *                           7 bits); 0 never; 1 wherever the matrix-core kernels apply.
  *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
  *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile

@@ -11,7 +11,10 @@
 // geometry
 // ---------------------------------------------------------------------------------------------------
 constexpr int KVC_WAVE = 64;               // lanes per tile = vectors per tile (include/kernels.h:13,18)
-constexpr int KVC_WAVES_PER_WG = 4;
+#ifndef KVC_WAVES_PER_WG_VALUE
+#define KVC_WAVES_PER_WG_VALUE 4
+#endif
+constexpr int KVC_WAVES_PER_WG = KVC_WAVES_PER_WG_VALUE;
 constexpr int KVC_WG = KVC_WAVE * KVC_WAVES_PER_WG;
 constexpr int KVC_V_TOKENS = 128;          // tokens per V vector (include/kernels.h:17)
 constexpr int KVC_MAX_TILE_BYTES = 8191;   // thread_info is u16 = end_byte*8 + pad (include/kernels.h:30-32)
@@ -24,7 +27,7 @@ constexpr int KVC_STAGE_WORDS = KVC_STAGE_BYTES / 4;
 // ---------------------------------------------------------------------------------------------------
 // decode look-up table (built on the device from the decode tree, see kvc_lut.hip)
 //
-//   header   {lbits, lmax, n_long, group, fused_group, fused_check, 0, 0}
+//   header   {lbits, lmax, n_long, group, fused_group, fused_check, OR of the symbols' fp16 bit patterns, 0}
 //   long[ ]  codes longer than lbits: {code left-aligned in 32 bits, len | sym << 8}
 //   entry[ ] 1 << lbits words indexed by the next lbits stream bits: len | sym << 8, or 0 when the
 //            code is longer than lbits (search long[]) or the bits match no code.
@@ -55,7 +58,7 @@ constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2
 // ---------------------------------------------------------------------------------------------------
 int kvc_fail(int code, const char *fmt, ...);
 // Tuning knobs settable through kvc_set_option (or, before first use, KVCOMP_<NAME> in the environment).
-enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_DECODE_PIPELINED = 5, KVC_OPT_FUSED_ROUNDED = 6, KVC_OPT_ATTENTION_TAIL_IN_MERGE = 7, KVC_OPT_COUNT };
+enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_DECODE_PIPELINED = 5, KVC_OPT_FUSED_ROUNDED = 6, KVC_OPT_ATTENTION_TAIL_IN_MERGE = 7, KVC_OPT_FUSED_MFMA = 8, KVC_OPT_COUNT };
 int kvc_option(KvcOption which);
 int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the

@@ -37,125 +37,12 @@
 // Slow path (codebooks with codes longer than the table index, tiles larger than the staging area, or
 // the rare overflow above): one symbol per refill, generic table read from global memory, payload read
 // from LDS or -- for an oversized tile -- from global memory.
-#include "kvc_tile.h"
-
-#include <mutex>
-#include <type_traits>
-
-struct KvcFusedArgs {
-    KvcStreamArgs s;
-    const int8_t *min_i8;
-    const __half *scale;
-    int quant_mask;
-    const __half *x;     // K: q [batch, q_heads, head_dim];  V: p [batch, q_heads, tokens]
-    void *out;           // K: scores [batch, q_heads, tokens]; V: partial [tokens/128, batch, q_heads, head_dim]
-    int out_f32;         // 0: fp16 (reference layout), 1: fp32
-    int64_t out_stride;  // K: elements between the score rows of two query heads (>= tokens)
-    // softmax kinds of the V kernel: instead of p it reads raw fp32 scores and forms, per 128-token group and
-    // query head, m = max(score * sm_scale), w = exp(score * sm_scale - m), l = sum w; the partial is the
-    // w-weighted sum and (m, l) go to ml[group][batch][q_head][2]
-    const float *scores;
-    int64_t scores_stride;
-    float sm_scale;
-    float *ml;
-    int64_t tokens;
-    int batch, kv_heads, q_heads, head_dim;
-    int table_words;     // LDS words reserved for the fused table (>= 1 << lbits of every codebook used)
-    int pack_words;      // LDS words per wave reserved for the packed tile payload (multiple of 4)
-    int pack_logical;    // payload words (lead words included) that fit there; fewer than pack_words when skewed
-    int skew;            // 0, or 2: every 32 payload words are followed by a copy of the next two (see kvc_skewed)
-    int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
-    int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
-    int double_window;   // refill 64 stream bits at a time where the vector length allows
-    // kvc_expand_kernel (plain decode, decode + dequantize): no x; the operand table holds {scale, min} per element
-    // Rounded mode of the matvec kernels: every (sym + min) * scale is rounded to fp16 before it meets q / p, as the
-    // reference's dequantizer does (models/cache/kvcomp_encode.py:146); the operand table then holds
-    // {min, scale, weight of each query head} per element and nothing is folded into a constant term.
-    int rounded;
-    int expand;          // 0: matvec kernels; 1: symbols out (uint8); 2: dequantized values out (fp16)
-    int out_words;       // LDS words per wave for the 32-element output slab
-};
-
-// Workgroups per CU (= waves per SIMD) each matvec kernel is compiled for.  With one query head per KV head the
-// decode loops wait on LDS round trips and every further wave pays, so those kernels get the most their register
-// demand allows without spilling (kinds 2 - 4 carry a second operand table or the softmax).  With four query heads
-// the four FMAs per symbol hide the round trip; measured, 4 and 5 waves tie and 6 or 7 are 6 - 8 % slower.
-constexpr int kvc_fused_occupancy(int rep, int kind)
-{
-    const bool two_slots = kind == 2 || kind == 4;
-    return rep == 1 ? (kind == 1 ? 8 : 7) : (rep == 2 || (rep == 4 && !two_slots)) ? 5 : 1;
-}
-#ifndef KVC_FUSED_OCC
-#define KVC_FUSED_OCC(REP, KIND) kvc_fused_occupancy(REP, KIND)
-#endif
-constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
-constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
-
-// What a tile needs from global memory, fetched into registers one tile ahead of its use.
-template <int REP, int SLOTS, int XW>
-struct KvcRaw {
-    uint4 pay[KVC_PRE_CHUNKS];        // payload chunks lane, lane + 64, ...
-    uint32_t off, bn;                 // block_info, clamped to the payload buffer (wave-uniform)
-    uint16_t ti_prev, ti_cur;         // thread_info of the previous lane (unused by lane 0) and of this lane
-    // operands of elements 2 * lane and 2 * lane + 1 (K: channels, V: tokens of the 128-token group), as loaded:
-    uint16_t sc[SLOTS][2];            // quantization scale (fp16 bits)
-    int8_t mn[SLOTS][2];              // quantization minimum
-    uint32_t x[SLOTS][REP][XW];       // per query head: q / p (two fp16 in one word), or two fp32 scores
-};
-// Nothing in it is touched before the tile is staged: any arithmetic on a loaded value would make the wave
-// wait for the load at that point and the fetch would no longer overlap the decode of the previous tile.
-
-// LDS traffic between the lanes of one wave needs no barrier (a wave's LDS operations complete in order);
-// this only keeps the compiler from moving accesses across the hand-over.
-__device__ __forceinline__ void kvc_wave_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// memory byte j of a word carries stream bits 8j .. 8j+7, most significant first: a byte swap followed by a
-// full bit reversal leaves stream bit k of the word at bit k
-__device__ __forceinline__ uint32_t kvc_stream_word(uint32_t raw) { return __brev(kvc_bswap(raw)); }
-
-// Skewed packed payload.  Lane l starts about l mean-stream-lengths into the payload, so when a small
-// multiple of that length is close to 32 words, every k-th lane reads the same bank at every refill.  With
-// two spare words after every 32 (holding a copy of the two words that follow, so that the three-word read
-// of a refill never has to jump), streams 32 words apart land two banks apart instead.
-//   word w of the payload lives at w + skew * (w >> 5), skew = 2 (or 0: plain layout)
-__device__ __forceinline__ uint32_t kvc_skewed(uint32_t w, uint32_t skew) { return __umul24(w >> 5, skew) + w; }
-
-// Byte address in LDS of payload word u >> 5 for a refill.  No clamp: a lane's position cannot pass its start
-// by more than 128 symbols x 10 bits, and the workgroup's LDS ends with that much slack (KVC_LDS_SLACK_WORDS),
-// so even a corrupt stream only ever reads this workgroup's own LDS.
-typedef __attribute__((address_space(3))) uint32_t kvc_lds_word;
-template <bool SKEW>
-__device__ __forceinline__ uint32_t kvc_refill_address(uint32_t stage_base, uint32_t u)
-{
-    const uint32_t a = u >> 5;
-    if (SKEW) return (a << 2) + (__umul24(u >> 10, 8u) + stage_base);     // + 2 words per 32
-    return (a << 2) + stage_base;
-}
-constexpr int KVC_LDS_SLACK_WORDS = 48;
-
-// Rounded mode: RN16((sym + min) * scale) as the reference's dequantizer computes it (sym + min exactly, one
-// rounding of the product).  Both steps are fp16 instructions: the sum of two small integers is exact in fp16
-// and an fp16 multiplication rounds the exact product once.  `ms` = {min, scale} as two fp16 in one word.
-__device__ __forceinline__ float kvc_rounded_value(__half sym, uint32_t ms)
-{
-    const __half mn = __ushort_as_half((unsigned short)(ms & 0xffffu)), sc = __ushort_as_half((unsigned short)(ms >> 16));
-    return __half2float(__hmul(__hadd(sym, mn), sc));
-}
+#include "kvc_fused_common.h"
 
 // -- slow path ----------------------------------------------------------------------------------------
 // One symbol per refill; table and long-code list in global memory; words from LDS (staged, bit-reversed)
 // or from global memory (raw, bounds-checked word by word).
 // Returns sum_i sym_i * ops[i * REP + r] for each query head r (ops: this lane's operand table in LDS).
-template <int REP>
-struct KvcVec {
-    float v[REP];
-};
-
 template <int REP, bool GSRC>
 __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_t nwords, uint32_t pos,
                                                   const uint32_t *__restrict__ lut_g, int n, const float *ops,
@@ -209,20 +96,6 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
 // `ops` is this lane's view of the wave's operand table in LDS: the same address in every lane (a broadcast
 // read) except in V tiles that straddle two heads, where the lanes of the second head point at its table.
 // Returns through `u` the new position and through `worst` the largest number of bits a group consumed.
-
-// LDS accessed by its byte offset: the table's offset is a multiple of its size, so "window bits | offset"
-// is the entry's address.
-typedef __attribute__((address_space(3))) uint32_t kvc_lds_u32;
-
-// compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>)
-template <int N, int I = 0, class Body>
-__device__ __forceinline__ void kvc_static_for(Body &&body)
-{
-    if constexpr (I < N) {
-        body(std::integral_constant<int, I>{});
-        kvc_static_for<N, I + 1>(body);
-    }
-}
 
 // acc += x * (the value of `quad` in lane (l & ~3) + J of lane l's quad): the lane permute rides on the FMA's
 // first operand, so picking one of the four operands a quad holds costs no instruction of its own.
@@ -392,116 +265,6 @@ __device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t &u,
     }
 }
 
-// -- tile geometry ------------------------------------------------------------------------------------
-// KIND 0: K tile (64 tokens x head_dim channels of one (batch, head); lane = token)
-// KIND 1: V tile (128 tokens x 64 flat channels; lane = channel), head_dim a multiple of 64: one head per tile
-// KIND 2: V tile with any other head_dim: the 64 channels may straddle two heads (two operand tables)
-// KIND 3, 4: as 1, 2 but with the softmax over the group's scores computed on the fly
-template <int KIND>
-struct KvcGeom {
-    static constexpr bool IS_K = KIND == 0;
-    static constexpr int SLOTS = (KIND == 2 || KIND == 4) ? 2 : 1;
-    static constexpr bool SOFTMAX = KIND >= 3;
-    static constexpr int XW = SOFTMAX ? 2 : 1;
-};
-
-// Issue the global loads of tile (row, col).  bi_off / bi_bn: the tile's block_info words.
-template <int REP, int KIND, int EXPAND = 0>
-__device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
-                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw)
-{
-    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
-    const int64_t tile = (int64_t)row * a.s.cols + col;
-    const int D = a.head_dim;
-    // sizes are clamped so that corrupt metadata yields wrong symbols, never an out-of-bounds access
-    uint32_t off = bi_off, bn = bi_bn & 0xffffu;
-    if (bn > (uint32_t)KVC_MAX_TILE_BYTES) bn = KVC_MAX_TILE_BYTES;
-    if ((int64_t)off >= a.s.enc_bytes) bn = 0;
-    else if ((int64_t)off + bn > a.s.enc_bytes) bn = (uint32_t)(a.s.enc_bytes - off);
-    raw.off = off;
-    raw.bn = bn;
-    const int64_t ti0 = tile * KVC_WAVE + lane;
-    raw.ti_prev = a.s.thread_infos[ti0 > 0 ? ti0 - 1 : 0];
-    raw.ti_cur = a.s.thread_infos[ti0];
-    // payload: whole aligned 16-byte chunks that each hold at least one payload byte (such reads never leave
-    // the pages the payload lives in)
-    const uint8_t *src = a.s.enc + off;
-    const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
-    const uint32_t nchunks = bn ? (head + bn + 15u) >> 4 : 0u;
-    const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
-#pragma unroll
-    for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
-        const uint32_t c = lane + 64 * j;
-        if (c < nchunks) raw.pay[j] = g[c];
-    }
-    // operands; lanes past the end of a short vector load the last pair (ignored when staged)
-    const uint16_t *scale16 = reinterpret_cast<const uint16_t *>(a.scale);
-    if (KIND == 0) {
-        const int b = col / a.kv_heads, h = col - b * a.kv_heads;
-        const int e0 = 2 * lane < D ? 2 * lane : D - 2;
-#pragma unroll
-        for (int half = 0; half < 2; half++) {
-            // per-channel pairs, or one pair per 64-token block (kernels.cu:771-772)
-            const int64_t g = a.quant_mask == KVC_MASK_CHANNEL ? tile * D + e0 + half : (int64_t)row;
-            if (EXPAND == 1) continue;                         // symbols out: no quantization parameters
-            raw.sc[0][half] = scale16[g];
-            raw.mn[0][half] = a.min_i8[g];
-        }
-        if (EXPAND == 0) {
-#pragma unroll
-            for (int r = 0; r < REP; r++)
-                raw.x[0][r][0] = *reinterpret_cast<const uint32_t *>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D + e0);
-        }
-    } else {
-        const int bh0 = (col * KVC_WAVE) / D;
-        const int bh_max = a.batch * a.kv_heads - 1;
-        const int64_t tk = (int64_t)row * KVC_V_TOKENS + 2 * lane;
-        const bool straddles = col * KVC_WAVE - bh0 * D + KVC_WAVE > D;   // wave-uniform
-#pragma unroll
-        for (int s = 0; s < SLOTS; s++) {
-            if (s == 1 && !straddles) continue;                // the second head's operands are not needed
-            int bh = bh0 + s;
-            bh = bh < bh_max ? bh : bh_max;                    // slot 1 is unused by a tile that ends the row
-            const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
-#pragma unroll
-            for (int half = 0; half < 2; half++) {
-                int64_t g;
-                if (a.quant_mask == KVC_MASK_V_TOKEN) g = tk + half;
-                else if (a.quant_mask == KVC_MASK_SIM_TOKEN) g = (tk + half) * a.batch + b;
-                else g = ((tk + half) * a.batch + b) * a.kv_heads + h;           // KVC_MASK_VECTOR
-                if (EXPAND == 1) continue;
-                raw.sc[s][half] = scale16[g];
-                raw.mn[s][half] = a.min_i8[g];
-            }
-#pragma unroll
-            for (int r = 0; r < REP; r++) {
-                if (EXPAND != 0) break;
-                const int64_t xrow = (int64_t)b * a.q_heads + h * REP + r;
-                if (KvcGeom<KIND>::SOFTMAX) {
-                    const uint2 v = *reinterpret_cast<const uint2 *>(a.scores + xrow * a.scores_stride + tk);
-                    raw.x[s][r][0] = v.x;
-                    raw.x[s][r][KvcGeom<KIND>::XW - 1] = v.y;
-                } else {
-                    raw.x[s][r][0] = *reinterpret_cast<const uint32_t *>(a.x + xrow * a.tokens + tk);
-                }
-            }
-        }
-    }
-}
-
-__device__ __forceinline__ float kvc_half_bits_to_float(uint32_t bits16)
-{
-    return __half2float(__ushort_as_half((unsigned short)bits16));
-}
-
-// What the decode step needs to know about a staged tile.
-struct KvcStaged {
-    bool fits;            // staged in LDS (wave-uniform); otherwise decode from global memory
-    uint32_t u0;          // fast-path start position (`lb` bits before the first code) in the lane's LDS words
-    const uint32_t *gwords;   // the lane's stream in global memory, from the aligned word holding its first byte
-    uint32_t gnwords, gpos;
-};
-
 // Move a fetched tile into LDS: payload -> packed area (-> per-lane rows), operands -> table; returns the
 // constant terms sum_i min_i * operand_i in bias[].
 template <int REP, int KIND, int EXPAND = 0>
@@ -512,56 +275,10 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     const int D = a.head_dim;
-    KvcStaged st;
-    // ---- payload
-    const uint32_t bn = raw.bn;
-    uint32_t start = lane ? (uint32_t)(raw.ti_prev >> 3) : 0u, end = (uint32_t)(raw.ti_cur >> 3);
-    if (start > bn) start = bn;
-    if (end > bn) end = bn;
-    if (end < start) end = start;
-    const uint8_t *src = a.s.enc + raw.off;
-    const uint32_t head = (uint32_t)(reinterpret_cast<uintptr_t>(src) & 15u);
-    const uint32_t nchunks = bn ? (head + bn + 15u) >> 4 : 0u;
-    const uint32_t first = head + start;                                   // byte offset in the packed area
-    const uint32_t nwords = end > start ? ((first & 3u) + (end - start) + 3u) >> 2 : 0u;
-    {
-        const uint8_t *lsrc = src + start;
-        const uint32_t skew = (uint32_t)(reinterpret_cast<uintptr_t>(lsrc) & 3u);
-        st.gwords = reinterpret_cast<const uint32_t *>(lsrc - skew);
-        st.gnwords = nwords;
-        st.gpos = skew * 8u;
-    }
-    // the packed area keeps row_words spare words at its end: the copy into rows below moves the same
-    // number of words for every lane, so the last lanes read past the payload
-    bool fits = KVC_PACK_LEAD + 4u * nchunks + 3u + (uint32_t)a.row_words <= (uint32_t)a.pack_logical;
-    uint32_t longest = 0;
-    if (a.row_words) {
-        longest = kvc_wave_max_dpp(nwords);
-        fits = fits && longest + 3u <= (uint32_t)a.row_words;
-    }
-    st.fits = fits;
-    if (fits) {
-        const uint32_t skew = (uint32_t)a.skew;
-        // chunk c holds payload words 4c .. 4c + 3 (after the lead words); chunks never straddle a run of 32
-        auto put = [&](uint32_t c, uint4 v) {
-            v.x = kvc_stream_word(v.x);
-            v.y = kvc_stream_word(v.y);
-            v.z = kvc_stream_word(v.z);
-            v.w = kvc_stream_word(v.w);
-            const uint32_t w = KVC_PACK_LEAD + 4u * c;
-            uint2 *dst = reinterpret_cast<uint2 *>(pack + kvc_skewed(w, skew));     // 8-byte aligned either way
-            dst[0] = make_uint2(v.x, v.y);
-            dst[1] = make_uint2(v.z, v.w);
-            if (skew && (w & 31u) == 0u) dst[-1] = make_uint2(v.x, v.y);           // the copy that ends the previous run
-        };
-#pragma unroll
-        for (int j = 0; j < KVC_PRE_CHUNKS; j++) {
-            const uint32_t c = lane + 64 * j;
-            if (c < nchunks) put(c, raw.pay[j]);
-        }
-        const uint4 *g = reinterpret_cast<const uint4 *>(src - head);
-        for (uint32_t c = lane + 64 * KVC_PRE_CHUNKS; c < nchunks; c += KVC_WAVE) put(c, g[c]);   // tiles beyond 4 KiB
-    }
+    uint32_t first, longest;
+    KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
+    const bool fits = st.fits;
+    const int pmode = kvc_pair_mode<KIND>(a);
     // ---- operand table: element i of head slot s, query head r at ops[(s * 128 + i) * REP + r]
     float bias_s[SLOTS][REP];
     const bool straddles = SLOTS == 2 && (col * KVC_WAVE) % D + KVC_WAVE > D;      // wave-uniform
@@ -576,8 +293,8 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 #pragma unroll
             for (int half = 0; half < 2; half++) {
                 const int i = 2 * lane + half;
-                const uint32_t mn_h = __half_as_ushort(__float2half_rn((float)raw.mn[s][half]));   // exact
-                ops[s * 128 + i] = __uint_as_float(mn_h | ((live ? (uint32_t)raw.sc[s][half] : 0u) << 16));
+                const uint32_t mn_h = __half_as_ushort(__float2half_rn((float)raw.min_int(s, half, pmode)));   // exact
+                ops[s * 128 + i] = __uint_as_float(mn_h | ((live ? raw.scale_bits(s, half, pmode) : 0u) << 16));
             }
             continue;
         }
@@ -608,12 +325,12 @@ __device__ __forceinline__ KvcStaged kvc_stage_tile(const KvcFusedArgs &a, int r
 #pragma unroll
         for (int half = 0; half < 2; half++) {
             const int i = 2 * lane + half;
-            const float sc = live ? kvc_half_bits_to_float(raw.sc[s][half]) : 0.f;
-            const float mn = (float)raw.mn[s][half];
+            const float sc = live ? kvc_half_bits_to_float(raw.scale_bits(s, half, pmode)) : 0.f;
+            const float mn = (float)raw.min_int(s, half, pmode);
             if (a.rounded) {                             // wave-uniform
                 float *o = ops + (s * 128 + i) * (REP + 1);
                 const uint32_t mn_h = __half_as_ushort(__float2half_rn(mn));                  // exact
-                o[0] = __uint_as_float(mn_h | ((live ? (uint32_t)raw.sc[s][half] : 0u) << 16));
+                o[0] = __uint_as_float(mn_h | ((live ? raw.scale_bits(s, half, pmode) : 0u) << 16));
 #pragma unroll
                 for (int r = 0; r < REP; r++) o[1 + r] = wgt[r][half];
                 continue;
@@ -1115,7 +832,7 @@ static void kvc_launch_fused(int kind, const KvcFusedArgs &a, dim3 grid, size_t 
 // from global memory, so the sizes only affect speed.  Everything stays within 64 KiB per workgroup.
 static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_bytes, int64_t tiles,
                            int64_t max_tile_bytes, int64_t max_stream_bytes, int max_code_bits, int64_t extra_words = 0,
-                           bool allow_pairs = true)
+                           bool allow_pairs = true, int64_t mfma_ops_words = 0)
 {
     const int force_rows = kvc_option(KVC_OPT_FUSED_ROWS);   // 0 / 1 overrides the choice below
     a.table_words = 1 << ((max_code_bits >= 1 && max_code_bits <= KVC_LUT_MAX_BITS) ? max_code_bits : KVC_LUT_MAX_BITS);
@@ -1129,9 +846,12 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
     if (allow_pairs && extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
         a.pair_bits = 2 * max_code_bits;
-        if (a.table_words < (2 << a.pair_bits)) a.table_words = 2 << a.pair_bits;
+        // eight bytes per entry (fp32 symbols), four in the matrix-core kernels (fp16 symbols)
+        const int words = (mfma_ops_words ? 1 : 2) << a.pair_bits;
+        if (a.table_words < words) a.table_words = words;
     }
-    const int64_t ops_words = (int64_t)slots * 128 * rep + extra_words;   // per wave, besides the payload
+    // per wave, besides the payload
+    const int64_t ops_words = mfma_ops_words ? mfma_ops_words : (int64_t)slots * 128 * rep + extra_words;
     const int64_t budget = (65536 / 4 - a.table_words - KVC_LDS_SLACK_WORDS) / KVC_WAVES_PER_WG - ops_words;   // words per wave
     const int64_t mean_tile = encoded_bytes / (tiles > 0 ? tiles : 1);
     // without the encoder's figure: tiles hold thousands of symbols, so their sizes stay close to the mean
@@ -1218,6 +938,8 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
         KVC_REQUIRE(quant_mask == KVC_MASK_V_TOKEN || quant_mask == KVC_MASK_SIM_TOKEN || quant_mask == KVC_MASK_VECTOR,
                     "fused V supports per-token quantization groups (0xE, 0xC, 0x8)");
     }
+    KVC_REQUIRE(((uintptr_t)d_scale & 3) == 0 && ((uintptr_t)d_min & 1) == 0,
+                "quant_scales must be 4-byte aligned and quant_min_ints 2-byte aligned");
     void *slot = nullptr;
     if (!d_luts) {
         if (int rc = kvc_workspace_slot(&slot)) return rc;
@@ -1249,8 +971,17 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     const int slots = (!is_k && head_dim % KVC_WAVE != 0) ? 2 : 1;
     const int kind = is_k ? 0 : (a.scores ? 2 : 0) + slots;
     const int rounded = kvc_option(KVC_OPT_FUSED_ROUNDED) != 0;
-    const size_t lds = kvc_plan_lds(a, slots, rounded ? (int)rep + 1 : (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes,
-                                    max_stream_bytes, max_code_bits, 0, !rounded);
+    // The matrix-core kernels take the common case: a codebook known to have codes of at most 7 bits, the plain or
+    // skewed packed payload, results that can be stored four at a time.
+    const int64_t out_stride = (extra && extra->out_stride) ? extra->out_stride : tokens;
+    const int want_mfma = kvc_option(KVC_OPT_FUSED_MFMA);
+    const bool mfma = (want_mfma < 0 ? rounded != 0 : want_mfma != 0) && max_code_bits >= 1 && max_code_bits <= 7 &&
+                      kvc_option(KVC_OPT_FUSED_ROWS) != 1 && ((uintptr_t)d_out & 15) == 0 &&
+                      (is_k ? out_stride % 4 == 0 : head_dim % 4 == 0);
+    const size_t lds = mfma ? kvc_plan_lds(a, slots, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes, max_stream_bytes,
+                                           max_code_bits, 0, true, kvc_mfma_ops_words(slots, (int)rep, rounded))
+                            : kvc_plan_lds(a, slots, rounded ? (int)rep + 1 : (int)rep, encoded_bytes, rows * a.s.cols,
+                                           max_tile_bytes, max_stream_bytes, max_code_bits, 0, !rounded);
     a.rounded = rounded;
     a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
     KvcTimer timer(elapsed_ms, stream);
@@ -1263,6 +994,12 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
         fprintf(stderr, "[kvcomp] fused kind %d rep %d: grid %u x %u, lds %zu B (table %d w, payload %d w of %d logical, "
                 "skew %d, rows %d), pair bits %d, tiles per wave %d, rounded %d\n", kind, (int)rep, grid.x, grid.y, lds,
                 a.table_words, a.pack_words, a.pack_logical, a.skew, a.row_words, a.pair_bits, a.s.tiles_per_wave, a.rounded);
+    if (mfma) {
+        if (trace_plan) fprintf(stderr, "[kvcomp]   matrix-core kernel\n");
+        kvc_launch_fused_mfma((int)rep, kind, rounded != 0, a, grid, lds, stream);
+        KVC_HIP(hipGetLastError());
+        return timer.finish();
+    }
     switch (rep) {
         case 1: kvc_launch_fused<1>(kind, a, grid, lds, stream); break;
         case 2: kvc_launch_fused<2>(kind, a, grid, lds, stream); break;
@@ -1287,6 +1024,8 @@ int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_t
         if (is_k && quant_mask != KVC_MASK_K_BLOCK && quant_mask != KVC_MASK_CHANNEL) return 1;
         if (!is_k && quant_mask != KVC_MASK_V_TOKEN && quant_mask != KVC_MASK_SIM_TOKEN && quant_mask != KVC_MASK_VECTOR) return 1;
     }
+    KVC_REQUIRE(!deq || (((uintptr_t)d_scale & 3) == 0 && ((uintptr_t)d_min & 1) == 0),
+                "quant_scales must be 4-byte aligned and quant_min_ints 2-byte aligned");
     void *slot = nullptr;
     if (int rc = kvc_workspace_slot(&slot)) return rc;
     KvcFusedArgs a;

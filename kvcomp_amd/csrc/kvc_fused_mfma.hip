@@ -1,0 +1,544 @@
+// kvc_fused_mfma.hip -- the fused decode + matvec kernels with the multiply-accumulate on the matrix cores.
+//
+//   kvc_fused_mfma_kernel<REP, 0, ROUNDED>      <- huffman_decode_and_mat_vec_mul   (kvcomp_cuda_extension/src/kernels.cu:721-776)
+//   kvc_fused_mfma_kernel<REP, 1 .. 4, ROUNDED> <- v_huffman_decode_and_mat_vec_mul (kernels.cu:778-861)
+//
+// Same work split, tile pipeline and lock-step table decode as kvc_fused.hip (one wave64 per tile, lane = stream, every
+// lane decodes element i of its stream at step i).  What differs is where the products are formed.  A lane keeps the
+// last four decoded elements as four fp16 in two registers, and one v_mfma_f32_4x4x4_16b_f16 multiplies them with the
+// wave-uniform operands of those four elements: the instruction computes, for each of its 16 blocks of four lanes,
+//   D[i][j] += sum_k A[i][k] B[k][j]        A[i][k]: element k of lane 4 block + i     (what the lane decoded)
+//                                           B[k][j]: held by lane 4 block + j          (operand column j)
+//                                           D[i][j]: register i of lane 4 block + j
+// so the 64 rows are the 64 lane streams (K: tokens, V: channels), k runs over four consecutive elements (K: channels,
+// V: tokens of the group) and the four columns are operand vectors.  Every query head owns two columns, the high and
+// the low fp16 part of its fp32 weight (the low part scaled by 4096, so both parts stay normal numbers): symbols are
+// exact in fp16, products of two fp16 are exact in the fp32 accumulator, and hi + lo / 4096 carries 22 bits of the
+// weight, so the result is as accurate as the fp32 FMA loop's.  One matrix instruction replaces 4 x REP FMAs, and the
+// operand comes from one 8-byte LDS read per lane (its own column: four addresses per wave).
+//
+// Rounded mode (KvcFusedArgs::rounded): every dequantized value is rounded to fp16 before it is multiplied, as the
+// reference's dequantizer rounds it (models/cache/kvcomp_encode.py:146): two elements at a time with one packed
+// fp16 add (sym + min, exact) and one packed fp16 multiply (one rounding of the exact product), the pairs of minima
+// and scales of a group of four elements arriving in one 16-byte broadcast read; the columns then hold q / the
+// softmax weights themselves.
+//
+// Tables: the one-symbol table holds {symbol as fp16, upper half; code length, lowest byte}.  Where twice the longest
+// code fits KvcFusedArgs::pair_bits and every symbol's fp16 pattern has its five lowest bits clear (symbols below 64,
+// and multiples of a power of two beyond), a two-symbol table {second symbol fp16 | first symbol fp16 | both lengths
+// in the lowest five bits} halves the look-ups; it is four bytes per entry, so it costs half the LDS cycles of an
+// eight-byte one.
+//
+// Everything that is not the common case (codes longer than 7 bits or than the table index, tiles that do not fit
+// the staging area) is decoded one symbol at a time by kvc_mfma_slow_tile, which reads the same operand tables.
+#include "kvc_fused_common.h"
+
+typedef _Float16 kvc_h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 kvc_h4 __attribute__((ext_vector_type(4)));
+typedef float kvc_f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t kvc_w2 __attribute__((ext_vector_type(2)));
+typedef uint32_t kvc_w4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) kvc_w2 kvc_lds_w2;
+typedef __attribute__((address_space(3))) kvc_w4 kvc_lds_w4;
+
+constexpr float KVC_LO_SCALE = 4096.f;
+constexpr uint32_t KVC_PAIR_LEN_MASK = 0x1fu;      // both code lengths of a two-symbol entry (at most 30)
+
+__device__ __forceinline__ uint32_t kvc_lds_addr(const void *p)
+{
+    return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
+}
+
+__device__ __forceinline__ kvc_f4 kvc_mfma4(uint32_t a01, uint32_t a23, kvc_w2 b, kvc_f4 c)
+{
+    const kvc_w2 a = {a01, a23};
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(kvc_h4, a), __builtin_bit_cast(kvc_h4, b), c, 0, 0, 0);
+}
+
+// {x.lo, x.hi} -> RN16((x + mn) * sc) per half: the sum of two small integers is exact in fp16, the product is
+// rounded once
+__device__ __forceinline__ uint32_t kvc_dequant_pair(uint32_t x, uint32_t mn, uint32_t sc)
+{
+    const kvc_h2 v = (__builtin_bit_cast(kvc_h2, x) + __builtin_bit_cast(kvc_h2, mn)) * __builtin_bit_cast(kvc_h2, sc);
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+// upper halves of two table entries side by side: {a >> 16, b >> 16 << 16}
+__device__ __forceinline__ uint32_t kvc_pack_hi16(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
+
+// -- operand tables -----------------------------------------------------------------------------------
+// btab  [slot][group g][set][column j][element k]  fp16: weight part of element 4 g + k for column 4 set + j;
+//       column 2 r is the high part of query head r's weight, column 2 r + 1 its low part times 4096
+// mstab [slot][group g] = {min 4g, min 4g+1 | min 4g+2, min 4g+3 | scale 4g, 4g+1 | scale 4g+2, 4g+3}  (rounded mode)
+template <int REP>
+struct KvcMfmaTables {
+    static constexpr int NM = kvc_mfma_sets(REP);
+    static constexpr int BTAB_SLOT_WORDS = KVC_MFMA_GROUPS * NM * 8;
+    static constexpr int MSTAB_SLOT_WORDS = KVC_MFMA_GROUPS * 4;
+};
+
+__device__ __forceinline__ uint32_t kvc_half_pair(float lo, float hi)
+{
+    return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
+}
+
+// Split v into a high fp16 part (zero where it would be subnormal) and the remainder times 4096 as fp16.
+__device__ __forceinline__ void kvc_split_weight(float v, float &hi, float &lo)
+{
+    const float h = __half2float(__float2half_rn(v));
+    hi = fabsf(h) < 6.103515625e-5f ? 0.f : h;
+    lo = (v - hi) * KVC_LO_SCALE;
+}
+
+// Build the operand tables of a fetched tile; returns per query head the constant term sum_i min_i weight_i of this
+// lane's head slot (zero in rounded mode) and the power of two the weights were divided by to stay inside fp16.
+template <int REP, int KIND, bool ROUNDED>
+__device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int row, int col, int lane,
+                                                   const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw,
+                                                   uint32_t *btab, uint32_t *mstab, float (&bias)[REP], float &unscale,
+                                                   int &sel_out)
+{
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    constexpr int NM = kvc_mfma_sets(REP);
+    using T = KvcMfmaTables<REP>;
+    const int D = a.head_dim;
+    float bias_s[SLOTS][REP];
+    float v[SLOTS][REP][2];
+    const bool straddles = SLOTS == 2 && (col * KVC_WAVE) % D + KVC_WAVE > D;      // wave-uniform
+    const bool live = KIND != 0 || 2 * lane < D;
+    const int pmode = kvc_pair_mode<KIND>(a);
+    float vmax = 0.f;
+#pragma unroll
+    for (int s = 0; s < SLOTS; s++) {
+#pragma unroll
+        for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f, v[s][r][0] = v[s][r][1] = 0.f;
+        if (s == 1 && !straddles) continue;                    // no lane of this tile belongs to a second head
+#pragma unroll
+        for (int r = 0; r < REP; r++) {
+            float w0, w1;                                      // the two elements' weights: q, p, or exp(score - max)
+            if (KvcGeom<KIND>::SOFTMAX) {
+                const float s0 = __uint_as_float(raw.x[s][r][0]) * a.sm_scale;
+                const float s1 = __uint_as_float(raw.x[s][r][KvcGeom<KIND>::XW - 1]) * a.sm_scale;
+                const float m = kvc_wave_fmax_dpp(fmaxf(s0, s1));
+                w0 = __expf(s0 - m);
+                w1 = __expf(s1 - m);
+                const float l = kvc_wave_sum_dpp(w0 + w1);
+                if (lane == 0) {
+                    int bh = (col * KVC_WAVE) / D + s;
+                    const int bh_max = a.batch * a.kv_heads - 1;
+                    bh = bh < bh_max ? bh : bh_max;
+                    const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
+                    float *ml = a.ml + (((int64_t)row * a.batch + b) * a.q_heads + h * REP + r) * 2;
+                    ml[0] = m;     // tiles that share a head write the same pair
+                    ml[1] = l;
+                }
+            } else {
+                w0 = kvc_half_bits_to_float(raw.x[s][r][0] & 0xffffu);
+                w1 = kvc_half_bits_to_float(raw.x[s][r][0] >> 16);
+            }
+            if (ROUNDED) {
+                v[s][r][0] = w0;
+                v[s][r][1] = w1;
+            } else {
+                const float sc0 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 0, pmode)) : 0.f;
+                const float sc1 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 1, pmode)) : 0.f;
+                v[s][r][0] = sc0 * w0;
+                v[s][r][1] = sc1 * w1;
+                bias_s[s][r] = (float)raw.min_int(s, 0, pmode) * v[s][r][0] + (float)raw.min_int(s, 1, pmode) * v[s][r][1];
+                vmax = fmaxf(vmax, fmaxf(fabsf(v[s][r][0]), fabsf(v[s][r][1])));
+            }
+        }
+        if (!ROUNDED) {
+#pragma unroll
+            for (int r = 0; r < REP; r++) bias_s[s][r] = kvc_wave_sum_dpp(bias_s[s][r]);
+        }
+    }
+    // weights beyond fp16's range (never with sane scales): divide the tile's weights by a power of two
+    float down = 1.f;
+    unscale = 1.f;
+    if (!ROUNDED && __any(!(vmax < 32768.f))) {
+        const float m = kvc_wave_fmax_dpp(vmax);
+        if (m < INFINITY) {                                    // otherwise the result is not finite either way
+            int e;
+            (void)frexpf(m, &e);                               // m < 2^e
+            down = ldexpf(1.f, 14 - e);
+            unscale = ldexpf(1.f, e - 14);
+        }
+    }
+    const int g = lane >> 1, odd = lane & 1;
+    if (live) {
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            if (s == 1 && !straddles) continue;
+#pragma unroll
+            for (int r = 0; r < REP; r++) {
+                float h0, l0, h1, l1;
+                kvc_split_weight(v[s][r][0] * down, h0, l0);
+                kvc_split_weight(v[s][r][1] * down, h1, l1);
+                const int c_hi = 2 * r, c_lo = 2 * r + 1;
+                uint32_t *bg = btab + s * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
+                bg[((c_hi >> 2) * 4 + (c_hi & 3)) * 2] = kvc_half_pair(h0, h1);
+                bg[((c_lo >> 2) * 4 + (c_lo & 3)) * 2] = kvc_half_pair(l0, l1);
+            }
+            if (ROUNDED) {
+                uint32_t *mg = mstab + s * T::MSTAB_SLOT_WORDS + g * 4 + odd;
+                mg[0] = kvc_half_pair((float)raw.min_int(s, 0, pmode), (float)raw.min_int(s, 1, pmode));           // exact
+                mg[2] = raw.scale_bits(s, 0, pmode) | (raw.scale_bits(s, 1, pmode) << 16);
+            }
+        }
+    }
+    int sel = 0;
+    if (SLOTS == 2) sel = ((col * KVC_WAVE) % D + lane) >= D;                 // 1 past a head boundary
+    sel_out = sel;
+#pragma unroll
+    for (int r = 0; r < REP; r++) bias[r] = (SLOTS == 2 && sel) ? bias_s[SLOTS - 1][r] : bias_s[0][r];
+}
+
+// -- decode loops -------------------------------------------------------------------------------------
+// 2 G symbols per refill of 64 stream bits (G from each half window; 2 G a multiple of four), n a multiple of 2 G.
+// bptr: LDS byte address of this lane's column in the operand table of the group the loop starts with;
+// msptr: of that group's minima and scales (rounded mode).  Both advance with the groups consumed.
+template <int G, bool SKEW, int NM, bool ROUNDED>
+__device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t mask4, int n,
+                                             uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM])
+{
+    static_assert((2 * G) % 4 == 0, "whole groups of four per refill");
+    for (int i = 0; i < n; i += 2 * G) {
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0;
+        uint32_t e[2 * G];
+        kvc_static_for<2 * G>([&](auto g_) {
+            constexpr int g = decltype(g_)::value;
+            if (g == G) R = __builtin_amdgcn_alignbit(hi, lo, es);
+            e[g] = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fe);
+            if (g != G - 1 && g != 2 * G - 1) R = __builtin_amdgcn_alignbit(R, R, e[g]);
+            es += e[g];
+            if constexpr (g % 4 == 3) {
+                constexpr int q = g / 4;
+                uint32_t a01 = kvc_pack_hi16(e[g - 3], e[g - 2]), a23 = kvc_pack_hi16(e[g - 1], e[g]);
+                if (ROUNDED) {
+                    const kvc_w4 ms = *(const kvc_lds_w4 *)(uintptr_t)(msptr + q * 16);
+                    a01 = kvc_dequant_pair(a01, ms.x, ms.z);
+                    a23 = kvc_dequant_pair(a23, ms.y, ms.w);
+                }
+#pragma unroll
+                for (int s = 0; s < NM; s++)
+                    acc[s] = kvc_mfma4(a01, a23, *(const kvc_lds_w2 *)(uintptr_t)(bptr + (q * NM + s) * 32), acc[s]);
+            }
+        });
+        u += es & 0xffu;
+        bptr += (2 * G / 4) * NM * 32;
+        msptr += (2 * G / 4) * 16;
+    }
+}
+
+// Two symbols per look-up: PG pairs from each half window, 4 PG symbols per refill; n a multiple of 4 PG.
+template <int PG, bool SKEW, int NM, bool ROUNDED>
+__device__ __forceinline__ void kvc_mfma_pair_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t maskp, int n,
+                                                  uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM])
+{
+    for (int i = 0; i < n; i += 4 * PG) {
+        const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
+        const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
+        const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
+        uint32_t R = lo, es = 0, used1 = 0;
+        uint32_t e[2 * PG];
+        kvc_static_for<2 * PG>([&](auto p_) {
+            constexpr int p = decltype(p_)::value;
+            if (p == PG) {
+                used1 = es & KVC_PAIR_LEN_MASK;                 // at most 30: the sum of a half window fits the field
+                R = __builtin_amdgcn_alignbit(hi, lo, used1);
+                es = 0;
+            }
+            e[p] = *(const kvc_lds_u32 *)(uintptr_t)((R & maskp) | fe);
+            if (p != PG - 1 && p != 2 * PG - 1) R = __builtin_amdgcn_alignbit(R, R, e[p]);
+            es += e[p];
+            if constexpr (p % 2 == 1) {
+                constexpr int q = p / 2;
+                uint32_t a01 = e[p - 1] & ~KVC_PAIR_LEN_MASK, a23 = e[p] & ~KVC_PAIR_LEN_MASK;
+                if (ROUNDED) {
+                    const kvc_w4 ms = *(const kvc_lds_w4 *)(uintptr_t)(msptr + q * 16);
+                    a01 = kvc_dequant_pair(a01, ms.x, ms.z);
+                    a23 = kvc_dequant_pair(a23, ms.y, ms.w);
+                }
+#pragma unroll
+                for (int s = 0; s < NM; s++)
+                    acc[s] = kvc_mfma4(a01, a23, *(const kvc_lds_w2 *)(uintptr_t)(bptr + (q * NM + s) * 32), acc[s]);
+            }
+        });
+        u += used1 + (es & KVC_PAIR_LEN_MASK);
+        bptr += PG * NM * 32;
+        msptr += PG * 16;
+    }
+}
+
+// One symbol per refill, generic table and long-code list in global memory; words from LDS (staged, bit-reversed)
+// or from global memory (raw, bounds-checked word by word).  Returns this lane's sums, one per query head.
+template <int REP, bool GSRC, bool ROUNDED>
+__device__ __noinline__ KvcVec<REP> kvc_mfma_slow_tile(const uint32_t *words, uint32_t nwords, uint32_t pos,
+                                                       const uint32_t *__restrict__ lut_g, int n, const uint32_t *btab,
+                                                       const uint32_t *mstab, uint32_t skew)
+{
+    constexpr int NM = kvc_mfma_sets(REP);
+    const uint32_t lshift = 32u - lut_g[0], nlong = lut_g[2];
+    const uint32_t *longs = lut_g + KVC_LUT_HEADER_WORDS;
+    const uint32_t *entries = lut_g + KVC_LUT_HEADER_WORDS + KVC_LUT_LONG_WORDS;
+    const uint16_t *bh = reinterpret_cast<const uint16_t *>(btab), *mh = reinterpret_cast<const uint16_t *>(mstab);
+    KvcVec<REP> acc;
+#pragma unroll
+    for (int r = 0; r < REP; r++) acc.v[r] = 0.f;
+    for (int i = 0; i < n; i++) {
+        const uint32_t wi = pos >> 5;
+        uint32_t w0 = 0, w1 = 0;
+        // either way the first stream bit of a word ends up in the most significant bit
+        if (wi < nwords) w0 = GSRC ? kvc_bswap(words[wi]) : __brev(words[kvc_skewed(wi, skew)]);
+        if (wi + 1 < nwords) w1 = GSRC ? kvc_bswap(words[wi + 1]) : __brev(words[kvc_skewed(wi + 1, skew)]);
+        const uint32_t hi = (uint32_t)(((((uint64_t)w0) << 32 | w1) << (pos & 31u)) >> 32);
+        const uint32_t e = entries[hi >> lshift];
+        uint32_t len = e & 0xffu, sym = (e >> 8) & 0xffu;
+        if (len == 0) {
+            len = 1;
+            sym = 0;
+            for (uint32_t j = 0; j < nlong; j++) {
+                const uint32_t c = longs[2 * j], ls = longs[2 * j + 1];
+                const uint32_t l = ls & 0xffu;
+                if (((hi ^ c) >> (32u - l)) == 0u) {
+                    len = l;
+                    sym = (ls >> 8) & 0xffu;
+                    break;
+                }
+            }
+        }
+        const int g = i >> 2, k = i & 3;
+        float x = (float)sym;
+        if (ROUNDED) {
+            const uint32_t ms = (uint32_t)mh[g * 8 + k] | ((uint32_t)mh[g * 8 + 4 + k] << 16);
+            x = kvc_rounded_value(__float2half_rn(x), ms);
+        }
+#pragma unroll
+        for (int r = 0; r < REP; r++) {
+            const int c_hi = 2 * r, c_lo = 2 * r + 1;
+            const float whi = kvc_half_bits_to_float(bh[((g * NM + (c_hi >> 2)) * 4 + (c_hi & 3)) * 4 + k]);
+            const float wlo = kvc_half_bits_to_float(bh[((g * NM + (c_lo >> 2)) * 4 + (c_lo & 3)) * 4 + k]);
+            acc.v[r] = fmaf(x, whi + wlo * (1.f / KVC_LO_SCALE), acc.v[r]);
+        }
+        pos += len;
+    }
+    return acc;
+}
+
+// value of `v` in the next lane of the quad (lanes 1 and 3 read themselves)
+__device__ __forceinline__ float kvc_quad_next(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xF5 /* quad_perm:[1,1,3,3] */, 0xf, 0xf, false));
+}
+
+template <int REP, int KIND, bool ROUNDED>
+__global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_mfma_kernel(KvcFusedArgs a)
+{
+    constexpr bool IS_K = KIND == 0;
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    constexpr int NM = kvc_mfma_sets(REP);
+    using T = KvcMfmaTables<REP>;
+    // dynamic LDS: the decode table (at offset 0, so that its address folds into the look-ups), then per wave:
+    // operand tables, packed payload
+    extern __shared__ __align__(16) uint32_t smem[];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int D = a.head_dim;
+    constexpr int OPS_WORDS = kvc_mfma_ops_words(SLOTS, REP, ROUNDED);
+    const int per_wave = OPS_WORDS + a.pack_words;
+    uint32_t *btab = smem + a.table_words + wave * per_wave;
+    uint32_t *mstab = btab + SLOTS * T::BTAB_SLOT_WORDS;
+    uint32_t *pack = btab + OPS_WORDS;
+    const int row = blockIdx.y;
+    const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
+    const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
+    const uint32_t lbits = lut_g[0], lmax = lut_g[1], nlong = lut_g[2];
+    const bool fast_book = nlong == 0 && lmax >= 1u && lmax <= 7u && (1u << lbits) <= (uint32_t)a.table_words;
+    // one-symbol entries: the symbol as fp16 in the upper half, the code length (never beyond the index width, which
+    // bounds how far a corrupt stream can run) in the lowest byte
+    auto fentry = [&](uint32_t i) {
+        const uint32_t e = lut_g[KVC_LUT_FENTRY_OFFSET + i];
+        const uint32_t len = (e & 0xffu) > lbits ? lbits : (e & 0xffu);
+        return ((uint32_t)__half_as_ushort(__float2half_rn(__uint_as_float(e & 0xffffff00u))) << 16) | len;
+    };
+    const uint32_t pbits = 2u * lmax;
+    // two symbols per look-up: twice the longest code fits the index, and no symbol's fp16 pattern needs the five
+    // bits the lengths of a two-symbol entry go to (header word 6: OR of all the patterns)
+    const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
+                       (1u << pbits) <= (uint32_t)a.table_words && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
+    if (pairs) {
+        // the one-symbol table goes to the (not yet used) per-wave areas; the two-symbol table is derived from it
+        uint32_t *tmp = smem + a.table_words;
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) tmp[i] = fentry(i);
+        __syncthreads();
+        const uint32_t m1 = (1u << lbits) - 1u;
+        for (uint32_t idx = tid; idx < (1u << pbits); idx += KVC_WG) {
+            const uint32_t e0 = tmp[idx & m1];
+            const uint32_t e1 = tmp[(idx >> (e0 & 0xffu)) & m1];
+            smem[idx] = (e1 & 0xffff0000u) | (e0 >> 16) | ((e0 & 0xffu) + (e1 & 0xffu));
+        }
+        __syncthreads();
+    } else if (fast_book) {
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) smem[i] = fentry(i);
+    }
+    // columns that no query head owns (REP 1: columns 2 and 3) are multiplied too: give them zeros once
+    for (int i = lane; i < SLOTS * T::BTAB_SLOT_WORDS; i += KVC_WAVE) btab[i] = 0;
+    if (lane < KVC_PACK_LEAD) pack[lane] = 0;
+    __syncthreads();
+    const uint32_t mask4 = ((1u << lbits) - 1u) << 2, maskp = ((1u << pbits) - 1u) << 2;
+    const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
+    // symbols per refill in the main part (a multiple of four); what is left goes eight per refill
+    const int per = pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
+    int n_main = (n / per) * per;
+    while ((n - n_main) % 8 != 0) n_main -= per;
+    const uint32_t fe = kvc_lds_addr(smem);                            // 0: the table opens the workgroup's LDS
+
+    // this wave's tiles: T consecutive columns of one tile row
+    const int TPW = a.s.tiles_per_wave;
+    const int col0 = (blockIdx.x * KVC_WAVES_PER_WG + wave) * TPW;
+    int ntiles = a.s.cols - col0;
+    ntiles = ntiles < TPW ? ntiles : TPW;
+    if (ntiles <= 0) return;
+    // block_info of tile col0 + j in lane j
+    uint32_t bi_off = 0, bi_bn = 0;
+    if (lane < ntiles) {
+        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.s.block_infos + 8 * ((int64_t)row * a.s.cols + col0 + lane));
+        bi_off = bi[0];
+        bi_bn = bi[1];
+    }
+    KvcRaw<REP, SLOTS, KvcGeom<KIND>::XW> raw;
+    kvc_fetch_tile<REP, KIND>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    float bias[REP], unscale;
+    int sel = 0;
+    uint32_t first, longest;
+    KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
+    if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;       // two bits before the lane's first code
+    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col0, lane, raw, btab, mstab, bias, unscale, sel);
+    kvc_wave_sync();
+    for (int it = 0; it < ntiles; it++) {
+        const int col = col0 + it;
+        const bool more = it + 1 < ntiles;
+        // the lane number is made opaque per tile, so that the addresses the fetch and the staging derive from it
+        // are not kept in registers through the decode loops
+        int lane_f = lane;
+        asm volatile("" : "+v"(lane_f));
+        if (more)   // loads for the next tile fly while this one is decoded
+            kvc_fetch_tile<REP, KIND>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
+                                      __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
+        const uint32_t *my_btab = btab + sel * T::BTAB_SLOT_WORDS, *my_mstab = mstab + sel * T::MSTAB_SLOT_WORDS;
+        // geometry of the results
+        int64_t out_base, out_step;
+        if (IS_K) {
+            const int b = col / a.kv_heads, h = col - b * a.kv_heads;
+            out_base = ((int64_t)b * a.q_heads + h * REP) * a.out_stride + (int64_t)row * KVC_WAVE;
+            out_step = a.out_stride;
+        } else {
+            const int c0 = col * KVC_WAVE;
+            const int bh0 = c0 / D, d0 = c0 - bh0 * D;                  // wave-uniform
+            const int b0 = bh0 / a.kv_heads, h0 = bh0 - b0 * a.kv_heads;
+            const int wrap = (h0 + sel == a.kv_heads) ? 1 : 0;          // the next head may open the next batch entry
+            const int b = b0 + wrap, h = wrap ? 0 : h0 + sel;
+            out_base = (((int64_t)row * a.batch + b) * a.q_heads + h * REP) * D + (d0 - sel * D);
+            out_step = D;
+        }
+        if (fast_book && st.fits) {
+            kvc_f4 acc[NM];
+#pragma unroll
+            for (int s = 0; s < NM; s++) acc[s] = kvc_f4{0.f, 0.f, 0.f, 0.f};
+            uint32_t u = st.u0;
+            uint32_t bptr = kvc_lds_addr(my_btab) + (lane & 3) * 8, msptr = kvc_lds_addr(my_mstab);
+            const uint32_t sbase = kvc_lds_addr(pack);
+            auto run = [&](auto skew_) {
+                constexpr bool SK = decltype(skew_)::value;
+                if (pairs) {
+                    if (per == 16) kvc_mfma_pair_dot<4, SK, NM, ROUNDED>(sbase, u, fe, maskp, n_main, bptr, msptr, acc);
+                    else kvc_mfma_pair_dot<3, SK, NM, ROUNDED>(sbase, u, fe, maskp, n_main, bptr, msptr, acc);
+                    if (n - n_main) kvc_mfma_pair_dot<2, SK, NM, ROUNDED>(sbase, u, fe, maskp, n - n_main, bptr, msptr, acc);
+                } else {
+                    if (per == 16) kvc_mfma_dot<8, SK, NM, ROUNDED>(sbase, u, fe, mask4, n_main, bptr, msptr, acc);
+                    else if (per == 12) kvc_mfma_dot<6, SK, NM, ROUNDED>(sbase, u, fe, mask4, n_main, bptr, msptr, acc);
+                    const int rest = per == 8 ? n : n - n_main;
+                    if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED>(sbase, u, fe, mask4, rest, bptr, msptr, acc);
+                }
+            };
+            if (a.skew) run(std::true_type{});
+            else run(std::false_type{});
+            // register i of lane 4 b + j: row 4 b + i, column 4 set + j; the even columns take their low parts from
+            // the lane to their right and carry the results of query head 2 set + j / 2
+            const int j = lane & 3, rows4 = (lane >> 2) * 4;
+#pragma unroll
+            for (int s = 0; s < NM; s++) {
+                float res[4];
+                const int r = 2 * s + (j >> 1);
+                float bs = 0.f;
+#pragma unroll
+                for (int rr = 0; rr < REP; rr++)
+                    if (rr == r) bs = bias[rr];
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    res[i] = fmaf(kvc_quad_next(acc[s][i]), 1.f / KVC_LO_SCALE, acc[s][i]) * unscale + bs;
+                if ((j & 1) == 0 && r < REP) {
+                    const int64_t o = out_base + r * out_step + rows4;
+                    if (a.out_f32) {
+                        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(a.out) + o) = make_float4(res[0], res[1], res[2], res[3]);
+                    } else {
+                        const uint32_t h01 = kvc_half_pair(res[0], res[1]), h23 = kvc_half_pair(res[2], res[3]);
+                        *reinterpret_cast<uint2 *>(reinterpret_cast<__half *>(a.out) + o) = make_uint2(h01, h23);
+                    }
+                }
+            }
+        } else {
+            KvcVec<REP> res;
+            if (st.fits)
+                res = kvc_mfma_slow_tile<REP, false, ROUNDED>(pack, (uint32_t)a.pack_logical, st.u0 + 2u, lut_g, n, my_btab,
+                                                              my_mstab, (uint32_t)a.skew);
+            else
+                res = kvc_mfma_slow_tile<REP, true, ROUNDED>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_btab, my_mstab, 0u);
+            // here a lane holds the results of its own row; in a V tile every lane's head slot is its block's
+#pragma unroll
+            for (int r = 0; r < REP; r++) {
+                const int64_t o = out_base + r * out_step + lane;
+                const float v = res.v[r] * unscale + bias[r];
+                if (a.out_f32) reinterpret_cast<float *>(a.out)[o] = v;
+                else reinterpret_cast<__half *>(a.out)[o] = __float2half(v);
+            }
+        }
+        if (more) {
+            kvc_wave_sync();     // every lane is done reading this tile's LDS data
+            int lane_s = lane;
+            asm volatile("" : "+v"(lane_s));
+            st = kvc_stage_payload(a, lane_s, raw, pack, first, longest);
+            if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;
+            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col + 1, lane_s, raw, btab, mstab, bias, unscale, sel);
+            kvc_wave_sync();
+        }
+    }
+}
+
+template <int REP, bool ROUNDED>
+static void kvc_launch_mfma_kind(int kind, const KvcFusedArgs &a, dim3 grid, size_t lds, hipStream_t stream)
+{
+    if (kind == 0) hipLaunchKernelGGL((kvc_fused_mfma_kernel<REP, 0, ROUNDED>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 1) hipLaunchKernelGGL((kvc_fused_mfma_kernel<REP, 1, ROUNDED>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 2) hipLaunchKernelGGL((kvc_fused_mfma_kernel<REP, 2, ROUNDED>), grid, dim3(KVC_WG), lds, stream, a);
+    else if (kind == 3) hipLaunchKernelGGL((kvc_fused_mfma_kernel<REP, 3, ROUNDED>), grid, dim3(KVC_WG), lds, stream, a);
+    else hipLaunchKernelGGL((kvc_fused_mfma_kernel<REP, 4, ROUNDED>), grid, dim3(KVC_WG), lds, stream, a);
+}
+
+void kvc_launch_fused_mfma(int rep, int kind, bool rounded, const KvcFusedArgs &a, dim3 grid, size_t lds, hipStream_t stream)
+{
+#define KVC_MFMA_REP(R)                                                         \
+    if (rounded) kvc_launch_mfma_kind<R, true>(kind, a, grid, lds, stream);     \
+    else kvc_launch_mfma_kind<R, false>(kind, a, grid, lds, stream)
+    switch (rep) {
+        case 1: KVC_MFMA_REP(1); break;
+        case 2: KVC_MFMA_REP(2); break;
+        case 4: KVC_MFMA_REP(4); break;
+        default: KVC_MFMA_REP(8); break;
+    }
+#undef KVC_MFMA_REP
+}

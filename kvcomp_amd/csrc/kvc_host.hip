@@ -51,8 +51,9 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"fused_double_window", "KVCOMP_FUSED_DOUBLE_WINDOW", 1},    // 64 stream bits per refill in the one-symbol loops
     {"fused_skew", "KVCOMP_FUSED_SKEW", -1},                     // skewed payload layout: -1 choose per call, 0 never, 1 always
     {"decode_pipelined", "KVCOMP_DECODE_PIPELINED", 1},          // plain decode / decode + dequantize on the fused kernels' machinery
-    {"fused_rounded", "KVCOMP_FUSED_ROUNDED", 0},                // 1: round each dequantized value to fp16 before the matvec (slower)
+    {"fused_rounded", "KVCOMP_FUSED_ROUNDED", 1},                // 1: round each dequantized value to fp16 before the matvec, as the reference's dequantizer does
     {"attention_tail_in_merge", "KVCOMP_ATTENTION_TAIL_IN_MERGE", 1},   // kvc_attention_decode: V's fp16 tail inside the merge kernel
+    {"fused_mfma", "KVCOMP_FUSED_MFMA", -1},                     // matrix-core kernels: -1 where they are faster (rounded mode), 0 never, 1 always
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;

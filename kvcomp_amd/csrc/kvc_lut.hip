@@ -20,6 +20,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
     __shared__ uint8_t s_bit[KVC_TREE_MAX_NODES];
     __shared__ uint32_t s_lmax, s_nlong;
     __shared__ float s_avg;   // sum over leaves of len * 2^-len: the mean code length if the code is well matched
+    __shared__ uint32_t s_symbits;   // OR over the symbols' fp16 patterns
 
     const int tid = threadIdx.x;
     const uint8_t *tree = trees + (int64_t)blockIdx.x * tree_stride;
@@ -27,7 +28,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
     int n_nodes = tree_bytes / node_bytes;
     if (n_nodes > KVC_TREE_MAX_NODES) n_nodes = KVC_TREE_MAX_NODES;
 
-    if (tid == 0) { s_lmax = 0; s_nlong = 0; s_avg = 0.f; }
+    if (tid == 0) { s_lmax = 0; s_nlong = 0; s_avg = 0.f; s_symbits = 0; }
     for (int n = tid; n < KVC_TREE_MAX_NODES; n += KVC_WG) {
         int leaf = 0, a = -1, b = -1;
         if (n < n_nodes) {
@@ -80,6 +81,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
                 my_code[k] = code;
                 atomicMax(&s_lmax, len);
                 atomicAdd(&s_avg, (float)len * exp2f(-(float)len));
+                atomicOr(&s_symbits, (uint32_t)__half_as_ushort(__float2half_rn((float)(s_child[0][n] & 0xff))));
             }
         }
     }
@@ -137,7 +139,7 @@ kvc_build_lut_kernel(const uint8_t *__restrict__ trees, int64_t tree_stride, int
         // enough for the window to overflow rarely (lut[5] = 1: the kernel checks and falls back)
         lut[4] = (lmax <= 3 || roomy8) ? 8u : lmax <= 7 ? 30u / lmax : roomy ? 4u : 2u;
         lut[5] = (roomy8 || (lmax > 7 && roomy)) ? 1u : 0u;
-        lut[6] = 0;
+        lut[6] = s_symbits;       // low bits clear in every symbol's fp16 pattern: room for lengths in a packed entry
         lut[7] = 0;
     }
 }

@@ -92,7 +92,7 @@ def test_entropy_encode_matches_oracle(shape, is_k):
 @pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((128, 2, 2, 128), 1), ((128, 2, 2, 128), 4), ((256, 1, 3, 64), 2),
                                        ((256, 2, 2, 96), 1), ((128, 1, 2, 96), 8)])
 @pytest.mark.parametrize("mask", [O.MASK_K_BLOCK, O.MASK_CHANNEL])
-def test_fused_k_matches_oracle(shape, rep, mask):
+def test_fused_k_matches_oracle(shape, rep, mask, fused_mode):
     T, B, H, D = shape
     x = S.synth_k(T, B, H, D)
     s = _make_stream(x, True, 0.1, mask, 64)
@@ -115,7 +115,7 @@ def test_fused_k_matches_oracle(shape, rep, mask):
 @pytest.mark.parametrize("shape,rep", [((256, 1, 4, 128), 1), ((256, 2, 2, 128), 1), ((256, 2, 2, 128), 4), ((128, 1, 3, 64), 2),
                                        ((256, 2, 2, 96), 1), ((128, 2, 4, 96), 2), ((128, 1, 2, 96), 8)])
 @pytest.mark.parametrize("mask", [O.MASK_V_TOKEN, O.MASK_SIM_TOKEN, O.MASK_VECTOR])
-def test_fused_v_matches_oracle(shape, rep, mask):
+def test_fused_v_matches_oracle(shape, rep, mask, fused_mode):
     T, B, H, D = shape
     x = S.synth_v(T, B, H, D)
     s = _make_stream(x, False, 0.2, mask, 128)
@@ -141,7 +141,7 @@ def test_quant_dequant_bit_exact(mask, eb):
 
 
 @pytest.mark.parametrize("eb_k,eb_v", [(0.3, 0.45), (0.03, 0.05)])
-def test_fused_across_code_length_regimes(eb_k, eb_v):
+def test_fused_across_code_length_regimes(eb_k, eb_v, fused_mode):
     """Short codes (8 symbols per window), and long codes (4 per window with the overflow check)."""
     m = kc()
     T, B, H, D = 256, 1, 4, 128
@@ -304,7 +304,7 @@ def test_errors_raise_instead_of_aborting():
 
 @pytest.mark.parametrize("is_k", [True, False])
 @pytest.mark.parametrize("nsym", [14, 22])
-def test_fused_with_long_codes_uses_slow_path(is_k, nsym):
+def test_fused_with_long_codes_uses_slow_path(is_k, nsym, fused_mode):
     """Codebooks whose codes exceed the table index: the fused kernels must fall back and still be right."""
     rng = np.random.default_rng(8)
     T, B, H, D = 256, 1, 2, 128
@@ -337,7 +337,7 @@ def test_fused_with_long_codes_uses_slow_path(is_k, nsym):
 
 
 @pytest.mark.parametrize("nsym,expect_lmax", [(200, 8), (12, 4), (7, 3)])
-def test_fused_k_window_groupings(nsym, expect_lmax):
+def test_fused_k_window_groupings(nsym, expect_lmax, fused_mode):
     """Near-uniform alphabets pin the code length, hence which window grouping the fused kernel takes:
     200 symbols -> 8-bit codes, too dense for four per window (two per refill); 12 -> 4-bit codes (four per
     refill, guaranteed); 7 -> 3-bit codes (eight per refill).  The 200-symbol book needs the int16 tree."""
@@ -368,7 +368,7 @@ def test_fused_k_window_groupings(nsym, expect_lmax):
 
 @pytest.mark.parametrize("D,rep", [(64, 1), (96, 1), (128, 1), (72, 1), (128, 4), (96, 2), (64, 8)])
 @pytest.mark.parametrize("nsym,expect_lmax", [(12, 4), (24, 5), (40, 6), (100, 7)])
-def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D, rep):
+def test_fused_group_sizes_and_remainders(nsym, expect_lmax, D, rep, fused_mode):
     """Exactly uniform alphabets give codes of 4 to 7 bits, for which a 30-bit half window is sure to hold 7, 6, 5
     and 4 symbols: the kernel decodes 14, 12, 10 or 8 symbols per refill and finishes a vector whose length is not
     a multiple of that with refills of 8 (head_dim 64, 72, 96 and 128; V vectors hold 128 symbols)."""

@@ -144,7 +144,7 @@ def test_smoke_entry():
 
 
 @pytest.mark.parametrize("k_mode,rep,extra", [("ChannelQuant", 1, 0), ("ChannelQuant", 4, 37), ("BlockQuant", 2, 200)])
-def test_compressed_attention_matches_fp32_reference(k_mode, rep, extra):
+def test_compressed_attention_matches_fp32_reference(k_mode, rep, extra, fused_mode):
     """Full decode attention (scores -> 1/sqrt(d) -> softmax -> p.V, grouped-query heads, uncompressed tails)
     against fp32 PyTorch attention over the dequantized cache: 1e-3 relative to max|out|."""
     from kvcomp_amd.ctx import KVCompCtx
@@ -162,12 +162,15 @@ def test_compressed_attention_matches_fp32_reference(k_mode, rep, extra):
     s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
     ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
     assert (out - ref).abs().max() <= 1e-3 * ref.abs().max()
+    # element by element: within 1e-3 of the value itself, or of the output's typical size for the smallest ones
+    if fused_mode.rounded:
+        assert torch.allclose(out, ref, rtol=1e-3, atol=1e-3 * float(ref.pow(2).mean().sqrt()))
 
 
 @pytest.mark.parametrize("rows", [0, 1])
 @pytest.mark.parametrize("tiles_per_wave", [1, 2, 3])
 @pytest.mark.parametrize("D", [128, 96])
-def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D):
+def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D, fused_mode):
     """The fused kernels may decode from the packed payload or from per-lane rows, and a wave may take one
     tile or a run of tiles (fetching one ahead): every combination must give the same attention output,
     including runs that are cut short at the end of a tile row (3 does not divide the tile columns)."""
@@ -194,16 +197,20 @@ def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D):
     kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
     s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
     ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
-    # the plan changes where the bits are read from, not the arithmetic: results are identical
-    assert torch.equal(out, default_plan)
-    # get() rounds every dequantized element to fp16, the fused kernels do not: the softmax turns that into
-    # a few 1e-3 of the output here
-    assert (out - ref).abs().max() <= 3e-3 * ref.abs().max()
+    # the plan changes where the bits are read from, not the arithmetic: results are identical, except that per-lane
+    # rows are only implemented by the fp32-FMA kernels, whose sums are rounded in a different order than the
+    # matrix cores' (both carry the products exactly)
+    same_kernel = rows == 0 or fused_mode.mfma == 0 or (fused_mode.mfma < 0 and not fused_mode.rounded)
+    if same_kernel:
+        assert torch.equal(out, default_plan)
+    else:
+        assert (out - default_plan).abs().max() <= 1e-5 * default_plan.abs().max()
+    assert (out - ref).abs().max() <= fused_mode.tol_vs_fp16_cache * ref.abs().max()
     assert L.kvc_set_option(b"no_such_option", 1) != 0
 
 
 @pytest.mark.parametrize("hint", ["too_small", "absent"])
-def test_compressed_attention_with_wrong_or_missing_size_hints(hint):
+def test_compressed_attention_with_wrong_or_missing_size_hints(hint, fused_mode):
     """The encoder's size hints only size the LDS staging: with hints that are too small (tiles do not fit and
     are decoded from global memory) or absent the result must not change."""
     from kvcomp_amd.ctx import KVCompCtx
@@ -226,7 +233,7 @@ def test_compressed_attention_with_wrong_or_missing_size_hints(hint):
 
 
 @pytest.mark.parametrize("T,D,rep,B", [(40, 128, 1, 1), (100, 128, 2, 2), (300, 64, 4, 1), (531, 96, 2, 2), (1024, 128, 8, 1)])
-def test_one_call_attention_matches_stepwise_and_fp32(T, D, rep, B):
+def test_one_call_attention_matches_stepwise_and_fp32(T, D, rep, B, fused_mode):
     """kvc_attention_decode (scores, per-group softmax, weighted values and the final merge inside the library)
     against the same result assembled step by step with PyTorch's softmax, and against fp32 attention over the
     dequantized cache.  Covers: nothing compressed yet, K compressed but V not, tails of different lengths."""
@@ -251,10 +258,10 @@ def test_one_call_attention_matches_stepwise_and_fp32(T, D, rep, B):
     kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
     s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
     ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
-    assert (out - ref).abs().max() <= 3e-3 * ref.abs().max()
+    assert (out - ref).abs().max() <= fused_mode.tol_vs_fp16_cache * ref.abs().max()
 
 
-def test_one_call_attention_grows_with_the_cache():
+def test_one_call_attention_grows_with_the_cache(fused_mode):
     """Prefill, then decode steps that push blocks out of the tails: attention after every few steps stays
     within tolerance of fp32 attention over what get() returns."""
     from kvcomp_amd.ctx import KVCompCtx
@@ -276,7 +283,7 @@ def test_one_call_attention_grows_with_the_cache():
             kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
             s = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
             ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s, dim=-1))
-            assert (out - ref).abs().max() <= 3e-3 * ref.abs().max(), "step %d" % i
+            assert (out - ref).abs().max() <= fused_mode.tol_vs_fp16_cache * ref.abs().max(), "step %d" % i
 
 
 @pytest.mark.parametrize("is_k,mode,B,H,D", [(True, "ChannelQuant", 2, 3, 96), (True, "BlockQuant", 1, 4, 128),
@@ -305,7 +312,7 @@ def test_one_kernel_get_equals_decode_then_dequant(is_k, mode, B, H, D):
     assert np.array_equal(one.cpu().numpy().view(np.uint16), deq.view(np.uint16))
 
 
-def test_attention_call_can_be_captured_in_a_graph():
+def test_attention_call_can_be_captured_in_a_graph(fused_mode):
     """kvc_attention_decode allocates nothing and waits for nothing, so a serving loop can record it in a HIP graph.
     The graph is replayed several times with eager work and synchronisations of the program's own in between, for
     queries that change between replays (the graph reads q and writes out in place), with and without fp16 tails;
