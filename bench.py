@@ -48,37 +48,34 @@ def log(*a):
 
 
 def make_kv(cfg, device, seed_offset=0):
-    """Synthetic K/V [T, B, H, D] fp16 generated on the device (seeded)."""
-    import torch
+    """Synthetic K/V [T, B, H, D] fp16 from the CPU-seeded generators the tests use (tests/_synth.py): generated in
+    fp32 on the host, cast to fp16, copied to the device, so that every run and the CPU oracle see the same bits."""
+    from tests import _synth as S
     T, B, H, D = cfg["T"], cfg["B"], cfg["H"], cfg["D"]
-    g = torch.Generator(device=device)
     if cfg["dist"] == "gauss":
-        g.manual_seed(1234 + 100 * seed_offset)
-        k = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32)
-        c = torch.exp(0.5 * torch.randn(H, D, generator=g, device=device, dtype=torch.float32))
-        g.manual_seed(1237)
-        for h in range(H):
-            c[h, torch.randperm(D, generator=g, device=device)[:4]] *= 20.0
-        k = (k * c).to(torch.float16)
-        g.manual_seed(1235 + 100 * seed_offset)
-        v = torch.randn(T, B, H, D, generator=g, device=device, dtype=torch.float32).to(torch.float16)
+        k = S.synth_k(T, B, H, D, seed=S.SEED_K + 100 * seed_offset)
+        v = S.synth_v(T, B, H, D, seed=S.SEED_V + 100 * seed_offset)
     else:
-        out = []
-        for seed in (1234, 1235):
-            g.manual_seed(seed)
-            u = torch.rand(T, B, H, D, generator=g, device=device, dtype=torch.float32) - 0.5
-            x = -torch.sign(u) * torch.log1p(-2.0 * u.abs().clamp(max=0.4999999))
-            m = torch.rand(T, B, H, D, generator=g, device=device) < 0.02
-            out.append(torch.where(m, x * 50.0, x).to(torch.float16))
-        k, v = out
-    return k, v
+        k = S.synth_laplace(T, B, H, D, S.SEED_K + 100 * seed_offset)
+        v = S.synth_laplace(T, B, H, D, S.SEED_V + 100 * seed_offset)
+    return k.to(device), v.to(device)
 
 
-def cpu_baseline(kctx, q, cfg, budget_s=12.0):
-    """The reference's fused K algorithm (bit-serial tree walk, fp16 dequantize, dot) restated in C
-    (oracle/kvc_oracle.c: kvo_fused_k_from_stream), timed on this host's cores over a bounded sample of
-    the same K stream."""
+def _sample_bytes(bi, nrows, cols, D, mask):
     import numpy as np
+    tiles = nrows * cols
+    payload = int(bi.view(np.uint32)[1::2][:tiles].astype(np.int64).sum())
+    groups = tiles * D if mask == 0x1 else nrows
+    return payload + tiles * 8 + tiles * 64 * 2 + groups * 3
+
+
+def cpu_baseline(kctx, q, k_fp16, cfg, budget_s=10.0):
+    """The reference's path restated on the host and timed on this machine's cores over bounded samples of the
+    same workload.  `value` is the fused K algorithm (bit-serial tree walk, fp16 dequantize, dot; oracle/kvc_oracle.c:
+    kvo_fused_k_from_stream) on all cores; `legs` adds the same on one thread, the reference's op-by-op PyTorch
+    quantizer (utils/compute.py:93-106) on the CPU, and its pure-Python heapq Huffman coder (utils/huffman.py)."""
+    import numpy as np
+    import torch
     from oracle import oracle as O
     from kvcomp_amd.compute import dims_to_mask
     B, H, D, T = cfg["B"], cfg["H"], cfg["D"], cfg["T"]
@@ -92,30 +89,57 @@ def cpu_baseline(kctx, q, cfg, budget_s=12.0):
     mask = dims_to_mask(kctx.quant_dims)
     stride, rows, cols = B * H * D, T // 64, B * H
     cores = int(os.environ.get("OMP_NUM_THREADS", "0")) or min(16, os.cpu_count() or 1)
+
+    def fused_leg(threads, budget):
+        O.lib().kvo_set_threads(threads)
+
+        def run(nrows):
+            t0 = time.perf_counter()
+            O.fused_k_from_stream(enc, bi, ti, tree, mn, sc, qh, nrows * 64, stride, vec_len=D, mask=mask)
+            return time.perf_counter() - t0
+
+        probe = max(1, min(rows, 2))
+        dt = run(probe)
+        nrows = int(max(probe, min(rows, probe * budget / max(dt, 1e-6))))
+        reps, total = 0, 0.0
+        while total < budget and reps < 200:          # repeat the bounded sample until ~budget seconds are timed
+            total += run(nrows)
+            reps += 1
+        return reps * _sample_bytes(bi, nrows, cols, D, mask) / total / 1e9, nrows, reps, total
+
+    gbs, nrows, reps, total = fused_leg(cores, budget_s)
+    out = {"value": round(gbs, 4), "unit": "GB/s", "cores": cores, "kind": "port",
+           "sample": "fused K (bit-serial tree-walk decode + fp16 dequant + dot, OpenMP over tiles) over the first %d of "
+                     "%d tokens of the same compressed K stream, %d passes, %.1f s" % (nrows * 64, T, reps, total)}
+    legs = {}
+    g1, n1, r1, t1 = fused_leg(1, 4.0)
+    legs["fused_k_single_thread"] = {"value": round(g1, 4), "unit": "GB/s compressed", "cores": 1,
+                                     "sample": "first %d tokens, %d passes, %.1f s" % (n1 * 64, r1, t1)}
     O.lib().kvo_set_threads(cores)
-
-    def run(nrows):
-        t0 = time.perf_counter()
-        O.fused_k_from_stream(enc, bi, ti, tree, mn, sc, qh, nrows * 64, stride, vec_len=D, mask=mask)
-        return time.perf_counter() - t0
-
-    def sample_bytes(nrows):
-        tiles = nrows * cols
-        payload = int(bi.view(np.uint32)[1::2][:tiles].astype(np.int64).sum())
-        per_group = D if mask == 0x1 else 1
-        groups = tiles * per_group if mask == 0x1 else nrows
-        return payload + tiles * 8 + tiles * 64 * 2 + groups * 3
-
-    probe = max(1, min(rows, 4))
-    dt = run(probe)
-    nrows = int(max(probe, min(rows, probe * budget_s / max(dt, 1e-6))))
-    reps, total = 0, 0.0
-    while total < budget_s and reps < 200:          # repeat the bounded sample until ~budget_s of CPU work is timed
-        total += run(nrows)
-        reps += 1
-    return {"value": round(reps * sample_bytes(nrows) / total / 1e9, 4), "unit": "GB/s", "cores": cores, "kind": "port",
-            "sample": "fused K (bit-serial tree-walk decode + fp16 dequant + dot, OpenMP over tiles) over the first %d of "
-                      "%d tokens of the same compressed K stream, %d passes, %.1f s" % (nrows * 64, T, reps, total)}
+    # the reference quantizer, one fp16 PyTorch op after the other (utils/compute.py:93-106), per-channel K groups
+    xs = k_fp16[:min(T, 2048)].cpu().reshape(-1, 64, B, H, D)
+    torch.set_num_threads(cores)
+    t0, n = time.perf_counter(), 0
+    while time.perf_counter() - t0 < 4.0:
+        mx, mi = xs.amax(dim=1, keepdim=True), xs.amin(dim=1, keepdim=True)
+        scale = (mx - mi) * cfg["eb_k"]
+        sym = (xs / scale).round() - (mi / scale).round()
+        n += 1
+    dt = time.perf_counter() - t0
+    legs["pytorch_cpu_quantizer"] = {"value": round(n * xs.numel() * 2 / dt / 1e9, 4), "unit": "GB/s fp16 in", "cores": cores,
+                                     "sample": "max/min/sub/mul/div/round/sub as separate fp16 CPU ops on the first %d tokens of K, "
+                                               "%d passes, %.1f s" % (xs.shape[0] * 64, n, dt)}
+    del sym
+    # the reference's whole-tensor Huffman coder (heapq tree + per-symbol string concatenation), 64 Ki symbols
+    syms = kctx.get_decode_quant_ints()[0].reshape(-1)[:65536].cpu().numpy()
+    t0 = time.perf_counter()
+    book = O.py_huffman_codebook(syms)
+    bits = O.py_bits(syms, book)
+    dt = time.perf_counter() - t0
+    legs["python_heapq_huffman"] = {"value": round(syms.size / dt / 1e9, 6), "unit": "GB/s symbols in", "cores": 1,
+                                    "sample": "65536 symbols of K, %d bits out, %.2f s (pure Python: not extrapolated)" % (bits.size, dt)}
+    out["legs"] = legs
+    return out
 
 
 def codec_rates(kctx, vctx, k, v, cfg):
@@ -169,18 +193,30 @@ def codec_rates(kctx, vctx, k, v, cfg):
     return out
 
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by
-# what the same counter reads for the 256 MiB kvc_calibration_copy_kernel of the same run (FETCH_SIZE x2.0,
-# WRITE_SIZE x1.0).  Source: profiles/fused_decode_attention_<workload>.md.
-MEASURED_TRAFFIC_BYTES = {
-    "cfg2": {"kvc_fused_kernel<1, 0>": int((4087.0 * 2.0 + 512.0) * 1024), "kvc_fused_kernel<1, 3>": int((2758.4 * 2.0 + 528.0) * 1024)},
-    "cfg3": {"kvc_fused_kernel<4, 0>": int((31971.0 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<4, 3>": int((26478.8 * 2.0 + 16640.0) * 1024)},
-    "cfg5": {"kvc_fused_kernel<1, 0>": int((102552.1 * 2.0 + 16384.0) * 1024), "kvc_fused_kernel<1, 4>": int((45746.0 * 2.0 + 12743.3) * 1024)},
-}
+def kernel_sources_digest():
+    """Digest of the kernel sources: measured counter figures are only quoted for the sources they were taken on."""
+    import hashlib
+    h = hashlib.sha256()
+    d = os.path.join(ROOT, "kvcomp_amd", "csrc")
+    for name in sorted(os.listdir(d)):
+        if name.endswith((".hip", ".h")):
+            with open(os.path.join(d, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
 
 
 def measured_traffic(workload, kernel):
-    return MEASURED_TRAFFIC_BYTES.get(workload, {}).get(kernel)
+    """HBM bytes per launch of `kernel` from profiles/traffic.json: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+    dispatch), each scaled by what the same counter reads for the 256 MiB kvc_calibration_copy_kernel of the same run.
+    None when the file has no figure for this kernel, or when it was measured on other kernel sources than these."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            t = json.load(f)
+    except (OSError, ValueError):
+        return None
+    if t.get("kernel_sources_digest") != kernel_sources_digest():
+        return None
+    return t.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
 def run_decode_loop(args):
@@ -329,8 +365,9 @@ def main():
     ap.add_argument("--workload", default=DEFAULT_WORKLOAD, choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--eb-k", type=float, default=None, help="override the K error bound of the workload (cfg5 sweeps 0.05 / 0.1 / 0.2)")
-    ap.add_argument("--no-rounded", action="store_true",
-                    help="skip the extra pass in rounded mode (keeps a kernel trace of this run to one variant per kernel)")
+    ap.add_argument("--no-unrounded", action="store_true",
+                    help="skip the extra pass in unrounded mode (keeps a kernel trace of this run to one variant per kernel)")
+    ap.add_argument("--no-sweep", action="store_true", help="cfg5: skip the sweep over K's error bound")
     ap.add_argument("--no-graph", action="store_true", help="skip the replay of the step as a captured HIP graph")
     ap.add_argument("--model-layers", type=int, default=0,
                     help="cfg4 only: run the Llama-2-7B architecture itself (random weights) with this many layers (32 = "
@@ -347,7 +384,9 @@ def main():
             "uses a second GPU (--gpus %d refused)" % args.gpus)
         sys.exit(2)
 
+    import copy
     import torch
+    from kvcomp_amd import _lib
     from kvcomp_amd.ctx import KVCompCtx, KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
     from kvcomp_amd import attention as A
 
@@ -360,19 +399,21 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     B, H, Hq, D, T = cfg["B"], cfg["H"], cfg["Hq"], cfg["D"], cfg["T"]
+    rep = Hq // H
     KVCompCacheConfigStatic.config = KVCompCacheConfig(args.workload, QuantMode.ChannelQuant, QuantMode.TokenQuant,
                                                        64, 128, 64, 128, cfg["eb_k"], cfg["eb_v"])
     log("[bench] %s" % cfg["desc"])
+    t0 = time.perf_counter()
     k, v = make_kv(cfg, dev)
+    log("[bench] inputs generated on the host (seeded) in %.1f s" % (time.perf_counter() - t0))
     kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    kctx.store(k)
-    vctx.store(v)
+    kctx.store(k, want_symbols=False)
+    vctx.store(v, want_symbols=False)
     torch.cuda.synchronize()
     t_store = time.perf_counter() - t0
     rates = codec_rates(kctx, vctx, k, v, cfg)
-    del k, v
     assert kctx.compressed_ctx_len == T and vctx.compressed_ctx_len == T
     kb, vb = kctx.compressed_bytes(), vctx.compressed_bytes()
     numel = T * B * H * D
@@ -380,13 +421,46 @@ def main():
         "(incl. codebook) %.1f ms" % (kb / 1e6, kctx.get_cr(), 8 * kctx.encoded_data.numel() / numel, vb / 1e6,
                                       vctx.get_cr(), 8 * vctx.encoded_data.numel() / numel, t_store * 1e3))
 
-    g = torch.Generator(device=dev).manual_seed(1236)
-    q = torch.randn(B, Hq, D, generator=g, device=dev, dtype=torch.float32).to(torch.float16)
-    attn = A.CompressedAttention(kctx, vctx)
+    g = torch.Generator().manual_seed(1236)
+    q = torch.randn(B, Hq, D, generator=g, dtype=torch.float32).to(torch.float16).to(dev)
+
+    # Several copies of the compressed cache, visited in turn, so that no step finds its stream in the 256 MiB
+    # last-level cache left there by the step before: the copies together hold at least 600 MB.
+    def cache_copies(kc, vc):
+        n = max(3, min(32, -(-600_000_000 // (kc.compressed_bytes() + vc.compressed_bytes()))))
+        return [A.CompressedAttention(kc, vc)] + [A.CompressedAttention(copy.deepcopy(kc), copy.deepcopy(vc)) for _ in range(n - 1)]
+
+    def time_steps(attns, steps, warmup):
+        """ms per step over `steps` steps between two synchronisations (the contract's figure), the per-step times
+        from events on the launch stream, and the mean durations of the two fused kernels from a second pass in
+        which the library brackets them by events of its own (that makes every call wait, so it is a pass apart)."""
+        out = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
+        n = len(attns)
+        for i in range(warmup):
+            attns[i % n].attend(q, out=out)
+        ev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            ev[i][0].record()
+            attns[i % n].attend(q, out=out)
+            ev[i][1].record()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+        per = sorted(a.elapsed_time(b) for a, b in ev)
+        pick = lambda f: per[min(len(per) - 1, int(f * len(per)))]
+        k_ms = v_ms = 0.0
+        for i in range(steps):
+            kms = []
+            attns[i % n].attend(q, out=out, kernel_ms=kms)
+            k_ms += kms[0] / steps
+            v_ms += kms[1] / steps
+        assert torch.isfinite(out).all()
+        return {"ms_per_step": ms, "event_ms": {"median": round(pick(0.5), 4), "p10": round(pick(0.1), 4), "p90": round(pick(0.9), 4)},
+                "k_ms": k_ms, "v_ms": v_ms, "out": out}
 
     if args.copy_calibration:
         import ctypes
-        from kvcomp_amd import _lib
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
         dst = torch.empty_like(src)
         _lib.check(_lib.lib().kvc_calibration_copy(ctypes.c_void_p(dst.data_ptr()), ctypes.c_void_p(src.data_ptr()),
@@ -394,50 +468,46 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    for _ in range(args.warmup):
-        attn.attend(q)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        out = attn.attend(q)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    ms_per_step = dt / args.steps * 1e3
-    # the same steps once more with the library bracketing its two fused kernels by events on the launch stream
-    # (that makes every call wait for them, so it is kept out of the step time above)
-    k_ms = v_ms = 0.0
-    for _ in range(args.steps):
-        ms = []
-        attn.attend(q, kernel_ms=ms)
-        k_ms += ms[0] / args.steps
-        v_ms += ms[1] / args.steps
-    log("[bench] step %.3f ms; fused K kernel %.3f ms (%.1f GB/s compressed), fused V kernel %.3f ms (%.1f GB/s compressed)"
-        % (ms_per_step, k_ms, kb / k_ms / 1e6, v_ms, vb / v_ms / 1e6))
-    assert torch.isfinite(out).all()
-    # the same pass in rounded mode: every dequantized value is rounded to fp16 before it meets q / p, as the
-    # reference's dequantizer rounds it (models/cache/kvcomp_encode.py:146)
-    from kvcomp_amd import _lib
-    rounded_ms = None
-    if not args.no_rounded:
-        was = _lib.set_option("fused_rounded", 1)
+    attns = cache_copies(kctx, vctx)
+    n_copies = len(attns)
+    # Before anything is timed: the operator against fp32 attention over the fp16 cache the reference's dequantizer
+    # gives (models/cache/kvcomp_encode.py:146), on one (batch, head) slice of this very cache, within 1e-3.
+    check = attns[0].attend(q)
+    kd = kctx.get_only_compressed()[0][:, 0, 0].float()
+    vd = vctx.get_only_compressed()[0][:, 0, 0].float()
+    for r in range(rep):
+        sref = torch.softmax((kd @ q[0, r].float()) / D ** 0.5, dim=0)
+        oref = sref @ vd
+        err = float((check[0, r] - oref).abs().max() / oref.abs().max())
+        assert err <= 1e-3, "decode attention differs from fp32 attention over the dequantized cache by %.2e" % err
+    del kd, vd
+    log("[bench] checked against fp32 attention over the dequantized cache (batch 0, KV head 0): max error %.1e of max|out|" % err)
+
+    res = time_steps(attns, args.steps, args.warmup)
+    ms_per_step, k_ms, v_ms = res["ms_per_step"], res["k_ms"], res["v_ms"]
+    log("[bench] step %.3f ms (events: median %.3f, p10 %.3f, p90 %.3f) over %d copies of the cache; fused K kernel %.3f ms "
+        "(%.1f GB/s compressed), fused V kernel %.3f ms (%.1f GB/s compressed)"
+        % (ms_per_step, res["event_ms"]["median"], res["event_ms"]["p10"], res["event_ms"]["p90"], len(attns), k_ms,
+           kb / k_ms / 1e6, v_ms, vb / v_ms / 1e6))
+    # the same pass with the dequantized values left unrounded (fp32 products; not the reference's cache values)
+    unrounded = None
+    if not args.no_unrounded:
+        was = _lib.set_option("fused_rounded", 0)
         try:
-            attn_r = A.CompressedAttention(kctx, vctx)
-            for _ in range(args.warmup):
-                attn_r.attend(q)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            for _ in range(args.steps):
-                attn_r.attend(q)
-            torch.cuda.synchronize()
-            rounded_ms = (time.perf_counter() - t0) / args.steps * 1e3
+            u = time_steps(attns, args.steps, args.warmup)
         finally:
             _lib.set_option("fused_rounded", was)
-        log("[bench] rounded mode: step %.3f ms" % rounded_ms)
+        unrounded = {"ms_per_step": round(u["ms_per_step"], 4), "GBs": round((kb + vb) / (u["ms_per_step"] * 1e-3) / 1e9, 1),
+                     "event_ms": u["event_ms"], "kernels_ms": {"fused_k": round(u["k_ms"], 4), "fused_v": round(u["v_ms"], 4)},
+                     "max_difference_from_default": float((u["out"] - res["out"]).abs().max() / res["out"].abs().max())}
+        log("[bench] unrounded mode: step %.3f ms; fused K %.3f ms, fused V %.3f ms" % (u["ms_per_step"], u["k_ms"], u["v_ms"]))
 
     # the same step captured once in a HIP graph and replayed (what a serving loop does with a launch-bound step:
     # the library call allocates nothing and waits for nothing, so it can be recorded as it is)
     graph_ms = None
     if not args.no_graph:
+        attn = attns[0]
+        out = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
         side = torch.cuda.Stream()
         with torch.cuda.stream(side):
             attn.attend(q, out=out)
@@ -456,41 +526,71 @@ def main():
         torch.cuda.synchronize()
         graph_ms = (time.perf_counter() - t0) / args.steps * 1e3
         assert torch.equal(out, eager), "graph replay differs from the eager call"
-        log("[bench] one step as a HIP graph, replayed: %.3f ms" % graph_ms)
+        log("[bench] one step as a HIP graph, replayed (one copy of the cache): %.3f ms" % graph_ms)
+
+    # cfg5 sweeps K's error bound (V fixed): one entry per bound, the same step on a cache compressed with it
+    sweep = None
+    if args.workload == "cfg5" and args.eb_k is None and not args.no_sweep:
+        sweep = []
+        for eb in (0.05, 0.1, 0.2):
+            at = None                                  # the previous bound's copies are released first
+            if eb == cfg["eb_k"]:
+                kc, at = kctx, attns
+            else:
+                kc = KVCompCtx(True, B, H, D, eb)
+                kc.store(k, want_symbols=False)
+                at = cache_copies(kc, vctx)
+            r = time_steps(at, args.steps, args.warmup)
+            bits = kc.max_code_bits
+            loop = ("matrix-core kernel, two symbols per look-up" if 2 * bits <= 8 else
+                    "matrix-core kernel, one symbol per look-up, %d per refill" % (16 if bits <= 3 else 12 if bits <= 5 else 8)
+                    if bits <= 7 else "fp32-FMA kernel, one symbol per look-up" if bits <= 10 else
+                    "fp32-FMA kernel, one symbol per refill (codes beyond the table index)")
+            sweep.append({"eb_k": eb, "ms_per_step": round(r["ms_per_step"], 4),
+                          "GBs": round((kc.compressed_bytes() + vb) / (r["ms_per_step"] * 1e-3) / 1e9, 1),
+                          "fused_k_ms": round(r["k_ms"], 4), "k_compressed_bytes": kc.compressed_bytes(),
+                          "k_bits_per_symbol": round(8 * kc.encoded_data.numel() / numel, 3), "k_max_code_bits": bits,
+                          "k_decode_loop": loop})
+            log("[bench] eb K %.2f: step %.3f ms, fused K %.3f ms, %.2f bits/sym, codes up to %d bits (%s)"
+                % (eb, r["ms_per_step"], r["k_ms"], sweep[-1]["k_bits_per_symbol"], bits, loop))
+    del k, v
 
     # template arguments: query heads per KV head, then 0 = K tile, 3 / 4 = V tile with the softmax on the fly
-    # (4: head_dim is not a multiple of 64, tiles may straddle two heads)
+    # (4: head_dim is not a multiple of 64, tiles may straddle two heads), then rounded mode
     v_kind = 3 if D % 64 == 0 else 4
-    dom, dom_ms, dom_bytes = (("kvc_fused_kernel<%d, 0>" % (Hq // H), k_ms, kb) if k_ms >= v_ms
-                              else ("kvc_fused_kernel<%d, %d>" % (Hq // H, v_kind), v_ms, vb))
+    mfma = kctx.max_code_bits <= 7, vctx.max_code_bits <= 7
+    name = lambda kind, m: ("kvc_fused_mfma_kernel<%d, %d, true>" % (rep, kind)) if m else ("kvc_fused_kernel<%d, %d>" % (rep, kind))
+    dom, dom_ms, dom_bytes = ((name(0, mfma[0]), k_ms, kb) if k_ms >= v_ms else (name(v_kind, mfma[1]), v_ms, vb))
     achieved = dom_bytes / dom_ms / 1e6
     value = (kb + vb) / (ms_per_step * 1e-3) / 1e9
     result = {
         "metric": "fused decompress-matvec GB/s (% HBM peak); Huffman enc/dec GB/s; comp ratio",
         "value": round(value, 3), "unit": "GB/s (compressed-cache bytes consumed per second by one decode-attention pass)",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 symbols, fp32 accumulate",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "u8 symbols, fp16 dequantized values, fp32 accumulate",
         "data": "synthetic", "config": {"workload": "%s: %s" % (args.workload, cfg["desc"]),
                                         "k_quant": "per-channel, 64-token blocks", "v_quant": "per-token",
                                         "compressed_bytes": {"k": kb, "v": vb}, "fp16_bytes_per_tensor": 2 * numel,
                                         "compression_ratio": {"k": round(kctx.get_cr(), 3), "v": round(vctx.get_cr(), 3)},
                                         "fp16_equivalent_GBs": round(4 * numel / (ms_per_step * 1e-3) / 1e9, 1),
                                         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
+                                        "event_ms_per_step": res["event_ms"], "cache_copies_cycled": n_copies,
                                         "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)},
-                                        "arithmetic": "q . ((sym + min) * scale) with the dequantized value kept in fp32 (within 1e-4 of "
-                                                      "fp64 attention over that dequantization); rounded_mode rounds it to fp16 first like "
-                                                      "the reference's dequantizer (within 1e-3 of fp32 attention over the fp16 cache)",
+                                        "arithmetic": "every (sym + min) * scale rounded to fp16 as the reference's dequantizer rounds it "
+                                                      "(models/cache/kvcomp_encode.py:146), fp32 accumulation: within 1e-3 of fp32 attention over "
+                                                      "that fp16 cache (checked in this run before timing); unrounded_mode keeps the products in fp32",
+                                        "check_max_error": err,
                                         "graph_replay_ms_per_step": None if graph_ms is None else round(graph_ms, 4),
-                                        "rounded_mode": None if rounded_ms is None else
-                                        {"ms_per_step": round(rounded_ms, 4), "GBs": round((kb + vb) / (rounded_ms * 1e-3) / 1e9, 1)},
+                                        "unrounded_mode": unrounded, "eb_k_sweep": sweep,
                                         "symbols_per_s": {"fused_k": round(numel / k_ms * 1e3), "fused_v": round(numel / v_ms * 1e3)},
-                                        "codec": rates},
+                                        "first_store_ms": round(t_store * 1e3, 2), "codec": rates},
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args.workload, dom)},
     }
     if not args.no_cpu_baseline:
-        log("[bench] timing the CPU restatement of the reference's fused K path ...")
-        result["cpu_baseline"] = cpu_baseline(kctx, q, cfg)
+        log("[bench] timing the CPU restatement of the reference's path ...")
+        k_head = make_kv(dict(cfg, T=min(T, 2048)), torch.device("cpu"))[0]
+        result["cpu_baseline"] = cpu_baseline(kctx, q, k_head, cfg)
     else:
         result["cpu_baseline"] = None
     print(json.dumps(result), flush=True)

@@ -49,10 +49,23 @@ __device__ __forceinline__ uint32_t kvc_lds_addr(const void *p)
     return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void *)p;
 }
 
+// BCAST: every block of four lanes takes its operand columns from lanes 0 - 15 (the instruction's lane-group pattern 4),
+// so only those sixteen lanes have to hold them.
+template <bool BCAST>
 __device__ __forceinline__ kvc_f4 kvc_mfma4(uint32_t a01, uint32_t a23, kvc_w2 b, kvc_f4 c)
 {
     const kvc_w2 a = {a01, a23};
+    if (BCAST) return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(kvc_h4, a), __builtin_bit_cast(kvc_h4, b), c, 0, 0, 4);
     return __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(kvc_h4, a), __builtin_bit_cast(kvc_h4, b), c, 0, 0, 0);
+}
+
+// This lane's operand columns of one group: an 8-byte LDS read, by the first sixteen lanes only where they serve all.
+template <bool BCAST>
+__device__ __forceinline__ kvc_w2 kvc_read_columns(uint32_t addr, bool holder)
+{
+    kvc_w2 b = {0u, 0u};
+    if (!BCAST || holder) b = *(const kvc_lds_w2 *)(uintptr_t)addr;
+    return b;
 }
 
 // {x.lo, x.hi} -> RN16((x + mn) * sc) per half: the sum of two small integers is exact in fp16, the product is
@@ -198,9 +211,9 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
 // 2 G symbols per refill of 64 stream bits (G from each half window; 2 G a multiple of four), n a multiple of 2 G.
 // bptr: LDS byte address of this lane's column in the operand table of the group the loop starts with;
 // msptr: of that group's minima and scales (rounded mode).  Both advance with the groups consumed.
-template <int G, bool SKEW, int NM, bool ROUNDED>
+template <int G, bool SKEW, int NM, bool ROUNDED, bool BCAST>
 __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t mask4, int n,
-                                             uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM])
+                                             uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM], bool holder)
 {
     static_assert((2 * G) % 4 == 0, "whole groups of four per refill");
     for (int i = 0; i < n; i += 2 * G) {
@@ -225,7 +238,7 @@ __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32
                 }
 #pragma unroll
                 for (int s = 0; s < NM; s++)
-                    acc[s] = kvc_mfma4(a01, a23, *(const kvc_lds_w2 *)(uintptr_t)(bptr + (q * NM + s) * 32), acc[s]);
+                    acc[s] = kvc_mfma4<BCAST>(a01, a23, kvc_read_columns<BCAST>(bptr + (q * NM + s) * 32, holder), acc[s]);
             }
         });
         u += es & 0xffu;
@@ -235,9 +248,9 @@ __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32
 }
 
 // Two symbols per look-up: PG pairs from each half window, 4 PG symbols per refill; n a multiple of 4 PG.
-template <int PG, bool SKEW, int NM, bool ROUNDED>
+template <int PG, bool SKEW, int NM, bool ROUNDED, bool BCAST>
 __device__ __forceinline__ void kvc_mfma_pair_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t maskp, int n,
-                                                  uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM])
+                                                  uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM], bool holder)
 {
     for (int i = 0; i < n; i += 4 * PG) {
         const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
@@ -265,7 +278,7 @@ __device__ __forceinline__ void kvc_mfma_pair_dot(uint32_t sbase, uint32_t &u, u
                 }
 #pragma unroll
                 for (int s = 0; s < NM; s++)
-                    acc[s] = kvc_mfma4(a01, a23, *(const kvc_lds_w2 *)(uintptr_t)(bptr + (q * NM + s) * 32), acc[s]);
+                    acc[s] = kvc_mfma4<BCAST>(a01, a23, kvc_read_columns<BCAST>(bptr + (q * NM + s) * 32, holder), acc[s]);
             }
         });
         u += used1 + (es & KVC_PAIR_LEN_MASK);
@@ -452,17 +465,20 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_mf
             uint32_t u = st.u0;
             uint32_t bptr = kvc_lds_addr(my_btab) + (lane & 3) * 8, msptr = kvc_lds_addr(my_mstab);
             const uint32_t sbase = kvc_lds_addr(pack);
+            // one head per tile: all sixteen blocks share their operand columns, which lanes 0 - 15 then hold for all
+            constexpr bool BCAST = SLOTS == 1;
+            const bool holder = lane < 16;
             auto run = [&](auto skew_) {
                 constexpr bool SK = decltype(skew_)::value;
                 if (pairs) {
-                    if (per == 16) kvc_mfma_pair_dot<4, SK, NM, ROUNDED>(sbase, u, fe, maskp, n_main, bptr, msptr, acc);
-                    else kvc_mfma_pair_dot<3, SK, NM, ROUNDED>(sbase, u, fe, maskp, n_main, bptr, msptr, acc);
-                    if (n - n_main) kvc_mfma_pair_dot<2, SK, NM, ROUNDED>(sbase, u, fe, maskp, n - n_main, bptr, msptr, acc);
+                    if (per == 16) kvc_mfma_pair_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, maskp, n_main, bptr, msptr, acc, holder);
+                    else kvc_mfma_pair_dot<3, SK, NM, ROUNDED, BCAST>(sbase, u, fe, maskp, n_main, bptr, msptr, acc, holder);
+                    if (n - n_main) kvc_mfma_pair_dot<2, SK, NM, ROUNDED, BCAST>(sbase, u, fe, maskp, n - n_main, bptr, msptr, acc, holder);
                 } else {
-                    if (per == 16) kvc_mfma_dot<8, SK, NM, ROUNDED>(sbase, u, fe, mask4, n_main, bptr, msptr, acc);
-                    else if (per == 12) kvc_mfma_dot<6, SK, NM, ROUNDED>(sbase, u, fe, mask4, n_main, bptr, msptr, acc);
+                    if (per == 16) kvc_mfma_dot<8, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
+                    else if (per == 12) kvc_mfma_dot<6, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
                     const int rest = per == 8 ? n : n - n_main;
-                    if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED>(sbase, u, fe, mask4, rest, bptr, msptr, acc);
+                    if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                 }
             };
             if (a.skew) run(std::true_type{});

@@ -101,7 +101,7 @@ class KVCompCacheConfigStatic:
 
 
 class _Growable:
-    """Device buffer that grows geometrically along dim 0; `.view` is the filled prefix."""
+    """Device buffer that grows geometrically (by a quarter) along dim 0; `.view` is the filled prefix."""
 
     def __init__(self):
         self.data: Optional[torch.Tensor] = None
@@ -109,11 +109,13 @@ class _Growable:
 
     def append(self, t: torch.Tensor):
         n = t.shape[0]
+        # room for a quarter more than is needed: re-allocation stays rare while decoding appends small pieces, and a
+        # context never holds much more than its stream
         if self.data is None:
-            cap = max(2 * n, 1)
+            cap = n + max(n // 4, 16)
             self.data = torch.empty((cap,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
         elif self.used + n > self.data.shape[0]:
-            cap = max(2 * self.data.shape[0], self.used + n)
+            cap = self.used + n + max((self.used + n) // 4, 16)
             grown = torch.empty((cap,) + tuple(self.data.shape[1:]), dtype=self.data.dtype, device=self.data.device)
             grown[:self.used] = self.data[:self.used]
             self.data = grown
@@ -182,7 +184,9 @@ class KVCompCtx:
     def _tail_append(self, cache: torch.Tensor):
         n = cache.shape[0]
         if self._tail is None or self._tail_len + n > self._tail.shape[0]:
-            cap = max(2 * (self._tail_len + n), self.block_size + self.recent_size + 64)
+            # what a context keeps between stores is less than block_size + recent_size tokens; room for that plus
+            # the tokens being appended (single tokens while decoding), with some slack against re-allocation
+            cap = self._tail_len + n + self.block_size + 64
             grown = torch.empty((cap,) + tuple(cache.shape[1:]), dtype=cache.dtype, device=cache.device)
             if self._tail_len:
                 grown[:self._tail_len] = self._tail[:self._tail_len]
@@ -231,35 +235,63 @@ class KVCompCtx:
         if self.device is None:
             self.device = cache.device
         assert self.device == cache.device, "device mismatch"
-        self.ctx_len += cache.shape[0]
-        # cut_tensor_ctx_len_0 (utils/compute.py:59-72) without re-allocating the tail on every call: append in
-        # place, then the leading whole blocks that leave the tail are compressed and the rest moves to the front
-        self._tail_append(cache)
-        n_blocks = blocks_to_compress(self._tail_len, self.block_size, self.recent_size)
+        # cut_tensor_ctx_len_0 (utils/compute.py:59-72): the leading whole blocks of (tail + new tokens) that leave the
+        # recent window are compressed, the rest is the new tail.  The blocks are taken from where they lie (the tail,
+        # the incoming tensor, or -- when they span both -- a copy of just those tokens), so a long prompt never passes
+        # through the tail and the tail stays a few blocks long.  Nothing of the context changes before the encoder
+        # has succeeded: a failed store (a symbol without a code, a tile beyond 8191 bytes) leaves it as it was.
+        n_new = cache.shape[0]
+        n_blocks = blocks_to_compress(self._tail_len + n_new, self.block_size, self.recent_size)
         if n_blocks <= 0:
+            self._tail_append(cache)
+            self.ctx_len += n_new
             return None
-        to_compress = self._tail[:n_blocks * self.block_size]
+        n_c = n_blocks * self.block_size
+        from_tail = min(n_c, self._tail_len)
+        if from_tail == 0:
+            to_compress = cache[:n_c].contiguous()
+        elif from_tail == n_c:
+            to_compress = self._tail[:n_c]
+        else:
+            to_compress = torch.cat([self._tail[:from_tail], cache[:n_c - from_tail]], dim=0)
+        sym = self._compress(to_compress, want_symbols)
+        if n_c >= self._tail_len:
+            rest = cache[n_c - self._tail_len:]
+            self._tail_len = 0
+            self._tail_append(rest)
+        else:
+            self._tail_drop_front(n_c)
+            self._tail_append(cache)
+        self.ctx_len += n_new
+        return sym
+
+    def _compress(self, to_compress: torch.Tensor, want_symbols: bool):
+        """Quantize + encode whole blocks [n * block_size, B, H, D] and append the stream; returns the symbols on the
+        two-step path.  State is only touched after the library calls have succeeded."""
         mask = dims_to_mask(self.quant_dims)
         if (not want_symbols and KVCompCtx.fused_store and self.encode_codebook is not None
                 and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
             self._store_fused(to_compress, mask)
-            self._tail_drop_front(n_blocks * self.block_size)
             return None
         blocked = to_compress.reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
         quant_ints, min_ints, quant_scale = quant(blocked, self.quant_dims, self.quant_scale_rel)
         sizes = kvcomp_cuda.calculate_buffer_size(quant_ints, self.is_k, self.head_num, self.head_dim)
         KVCompCtx.buffer_ctx_len[self.device] = to_compress.shape[0]
         bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
+        codebook = None
         if self.encode_codebook is None:     # first stored chunk defines the codebook (kvcomp_encode.py:99-103)
             if self.codebook_smoothing:
-                enc, dec = self._smoothed_codebook(quant_ints)
+                codebook = self._smoothed_codebook(quant_ints)
             else:
                 shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
                 assert shift == 0, "shift must be 0"
-            self._set_codebook(enc, dec)
+                codebook = (enc, dec)
+        enc_table = self.encode_codebook if codebook is None else codebook[0].to(self.device)
         fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
-        encoded_, block_infos_, vec_infos_ = fn(quant_ints, self.encode_codebook, bi_buf, ti_buf, idx_buf, payload_buf,
+        encoded_, block_infos_, vec_infos_ = fn(quant_ints, enc_table, bi_buf, ti_buf, idx_buf, payload_buf,
                                                 self._encoded.used, self.head_num, self.head_dim)
+        if codebook is not None:
+            self._set_codebook(*codebook)
         self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
         self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
         self._encoded.append(encoded_)
@@ -268,7 +300,6 @@ class KVCompCtx:
         self._min_ints.append(min_ints)
         self._scales.append(quant_scale)
         self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
-        self._tail_drop_front(n_blocks * self.block_size)
         return quant_ints
 
     # The reference derives the one codebook of a stream from its first stored chunk alone, so a symbol that first
@@ -414,6 +445,17 @@ class KVCompCtx:
     @property
     def shape(self):
         return torch.Size([self.compressed_ctx_len, self.batch_size, self.head_num, self.head_dim])
+
+    def held_bytes(self) -> int:
+        """Device memory this context holds, from the capacities of its buffers (not just their filled parts)."""
+        n = 0 if self._tail is None else self._tail.numel() * self._tail.element_size()
+        for g in (self._encoded, self._block_infos, self._thread_infos, self._min_ints, self._scales):
+            if g.data is not None:
+                n += g.data.numel() * g.data.element_size()
+        for t in (self.encode_codebook, self.decode_codebook):
+            if t is not None:
+                n += t.numel()
+        return n
 
     def compressed_bytes(self) -> int:
         """Denominator of get_cr (kvcomp_encode.py:318-324): everything a fused kernel has to read."""

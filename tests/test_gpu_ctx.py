@@ -118,6 +118,40 @@ def test_prefill_then_append_one_token_at_a_time():
     assert np.array_equal(ctx.get_decode_quant_ints()[0].cpu().numpy(), o[3])
 
 
+def test_a_context_holds_little_more_than_its_stream():
+    """After a long prompt the fp16 tail is a few blocks, not the prompt: device memory held (capacities, not just
+    the filled parts) stays well below the dense cache, and a failed store leaves the context unchanged."""
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd._lib import KvcompError
+    _config(k_mode="ChannelQuant")
+    T, B, H, D = 4096, 2, 4, 128
+    for is_k in (True, False):
+        x = (S.synth_k if is_k else S.synth_v)(T + 17, B, H, D).to(DEV)
+        ctx = KVCompCtx(is_k, B, H, D, 0.1 if is_k else 0.2)
+        ctx.store(x[:T], want_symbols=False)
+        for i in range(T, T + 17):
+            ctx.store(x[i:i + 1], want_symbols=False)
+        dense = 2 * (T + 17) * B * H * D
+        assert ctx._tail.shape[0] <= 2 * (ctx.block_size + ctx.recent_size) + 64
+        assert ctx.held_bytes() <= 0.45 * dense, (ctx.held_bytes(), dense)
+        assert ctx.held_bytes() >= ctx.compressed_bytes() + ctx.buffer.numel() * 2
+        full, _ = ctx.get()
+        assert torch.equal(full[ctx.compressed_ctx_len:], x[ctx.compressed_ctx_len:])
+    # a store whose encode fails (a symbol the codebook has no code for) changes nothing
+    _config(k_mode="BlockQuant")
+    ctx = KVCompCtx(True, 1, 2, 128, 0.1)
+    flat = torch.zeros(128, 1, 2, 128, dtype=torch.float16, device=DEV)
+    flat[::2] = 1.0                                               # two symbols only: 0 and 10
+    ctx.store(flat)
+    before = (ctx.ctx_len, ctx.compressed_ctx_len, ctx.buffer.shape[0], ctx.encoded_data.numel())
+    wide = S.synth_k(128, 1, 2, 128).to(DEV)                      # needs the symbols in between
+    with pytest.raises(KvcompError):
+        ctx.store(wide)
+    assert before == (ctx.ctx_len, ctx.compressed_ctx_len, ctx.buffer.shape[0], ctx.encoded_data.numel())
+    ctx.store(flat)                                               # and the context still works
+    assert ctx.ctx_len == 256
+
+
 def test_batch_and_gqa_heads():
     from kvcomp_amd.ctx import KVCompCtx
     _config(k_mode="ChannelQuant")
