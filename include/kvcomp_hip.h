@@ -155,6 +155,49 @@ int kvc_store_fused(int is_k, const void *d_x_f16, int64_t tokens, int64_t batch
                     uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap, uint32_t base_global_offset,
                     int64_t *h_total_bytes, int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream);
 
+/* ---- encode without a host round trip (no counterpart in the reference: its encoder copies its counters to the host
+ * and waits for the device on every call, kernels.cu:950-965, and takes one codebook per call) -------------------
+ * kvc_encode_async queues one encode (from symbols, or -- d_sym == NULL -- quantizing d_x_f16 on the fly exactly as
+ * kvc_store_fused does) and returns without waiting; nothing in it is a memset, so it can be recorded in a HIP graph.
+ *   codebooks   n tables as kvc_build_codebook_device writes them, table_stride_bytes apart; tile row r (64 tokens of K,
+ *               128 of V) is encoded with table r / rows_per_codebook (0: one table for every row).  With
+ *               d_codebook_meta (that builder's int32[n][4]) a table that was not built flags the call.
+ *   placement   d_stream_bytes == NULL: the payload goes to d_encoded[0 ..) and block_info.offset = base_global_offset +
+ *               position, as in kvc_k_/v_entropy_encode.  Otherwise *d_stream_bytes (device, in / out) says how many
+ *               payload bytes d_encoded already holds: the call appends behind them, offsets continue from there, and
+ *               on success the counter moves on -- so successive calls need no size from the host.
+ *   d_result    device uint32[8], zeroed once by the caller, then shared by successive calls:
+ *               [0] payload bytes of the latest call, [1] error bits of all calls so far (0 = none), [2] largest tile
+ *               payload and [3] longest lane stream so far (sizing hints of the fused decoders), [4] tiles encoded
+ *               so far, [5] block_info.offset of the latest call's first tile.
+ * kvc_encode_result copies d_result to the host (it waits for the stream), turns error bits into an error return
+ * and hands out the figures (any pointer may be NULL). */
+typedef struct kvc_encode_job {
+    int32_t is_k;
+    int32_t quant_mask;               /* d_sym == NULL: layout of the (min, scale) groups, as for kvc_store_fused */
+    const uint8_t *d_sym;             /* uint8 [tokens, batch * heads * head_dim], or NULL */
+    const void *d_x_f16;              /* d_sym == NULL: fp16 [tokens, batch, heads, head_dim] */
+    float eb;
+    int8_t *d_min_i8;                 /* d_sym == NULL: quantizer outputs */
+    void *d_scale_f16;
+    int64_t tokens, batch, heads, head_dim;
+    const uint8_t *d_encode_tables;
+    int64_t encode_table_bytes;       /* bytes of a table that hold entries (at most 2048) */
+    int64_t table_stride_bytes;
+    int64_t rows_per_codebook;
+    const int32_t *d_codebook_meta;   /* may be NULL */
+    uint8_t *d_block_infos;
+    uint8_t *d_thread_infos;
+    uint8_t *d_encoded;
+    int64_t encoded_cap;
+    uint32_t base_global_offset;
+    uint32_t *d_stream_bytes;         /* may be NULL */
+    uint32_t *d_result;               /* may be NULL if d_stream_bytes is not */
+} kvc_encode_job;
+int kvc_encode_async(const kvc_encode_job *job, void *stream);
+int kvc_encode_result(const uint32_t *d_result, int64_t encoded_cap, int64_t *h_total_bytes, int64_t *h_max_tile_bytes,
+                      int64_t *h_max_stream_bytes, int64_t *h_tiles, void *stream);
+
 /* ---- decode: k_/v_entropy_decode_cuda_export (kernels.cu:1013-1087) -------------------------------
  * d_out uint8 [tokens, stride].  If elapsed_ms != NULL the kernel is bracketed by events, the call
  * waits for it and stores the elapsed milliseconds (the reference's return value); otherwise the call

@@ -24,6 +24,18 @@ class CompressedDesc(C.Structure):
                 ("d_tail_f16", C.c_void_p), ("tail_tokens", C.c_int64)]
 
 
+class EncodeJob(C.Structure):
+    """kvc_encode_job of include/kvcomp_hip.h."""
+    _fields_ = [("is_k", C.c_int32), ("quant_mask", C.c_int32), ("d_sym", C.c_void_p), ("d_x_f16", C.c_void_p),
+                ("eb", C.c_float), ("d_min_i8", C.c_void_p), ("d_scale_f16", C.c_void_p),
+                ("tokens", C.c_int64), ("batch", C.c_int64), ("heads", C.c_int64), ("head_dim", C.c_int64),
+                ("d_encode_tables", C.c_void_p), ("encode_table_bytes", C.c_int64), ("table_stride_bytes", C.c_int64),
+                ("rows_per_codebook", C.c_int64), ("d_codebook_meta", C.c_void_p),
+                ("d_block_infos", C.c_void_p), ("d_thread_infos", C.c_void_p), ("d_encoded", C.c_void_p),
+                ("encoded_cap", C.c_int64), ("base_global_offset", C.c_uint32),
+                ("d_stream_bytes", C.c_void_p), ("d_result", C.c_void_p)]
+
+
 # name -> argtypes (every function returns int unless listed in _RESTYPES)
 _SIGNATURES = {
     "kvc_abi_version": [],
@@ -40,6 +52,8 @@ _SIGNATURES = {
     "kvc_store_fused_supported": [_int, _int, _i64, _i64, _i64],
     "kvc_store_fused": [_int, _vp, _i64, _i64, _i64, _i64, _int, C.c_float, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _i64,
                         _u32, _i64p, _i64p, _i64p, _vp],
+    "kvc_encode_async": [C.POINTER(EncodeJob), _vp],
+    "kvc_encode_result": [_vp, _i64, _i64p, _i64p, _i64p, _i64p, _vp],
     "kvc_k_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_v_entropy_decode": [_vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _i64, _i64, _i64, _i64, _f32p, _vp],
     "kvc_decode_dequant": [_int, _vp, _i64, _vp, _i64, _vp, _i64, _vp, _i64, _int, _vp, _vp, _int, _i64, _vp, _i64, _i64, _i64,

@@ -113,7 +113,8 @@ class CompressedAttention:
             d.d_luts = lut.data_ptr()
             d.d_block_infos, d.block_infos_bytes = ctx.block_infos.data_ptr(), ctx.block_infos.numel()
             d.d_thread_infos, d.thread_infos_bytes = ctx.thread_infos.data_ptr(), ctx.thread_infos.numel()
-            d.d_encoded, d.encoded_bytes = ctx.encoded_data.data_ptr(), ctx.encoded_data.numel()
+            enc, enc_bytes = ctx.encoded_nosync()          # an address and a bound: no wait for queued encodes
+            d.d_encoded, d.encoded_bytes = enc.data_ptr(), enc_bytes
             d.d_quant_min_ints, d.d_quant_scales_f16 = ctx.quant_min_ints.data_ptr(), ctx.quant_scales.data_ptr()
         d.rows_per_codebook = 0
         d.quant_mask = dims_to_mask(ctx.quant_dims)

@@ -166,6 +166,7 @@ class KVCompCacheCuda:
         self.v_cache_buffer = [KVCompCtx(False, batch_size, head_num, head_dim, cfg.v_quant_scale_rel) for _ in range(layer_num)]
         for ctx in self.k_cache_buffer + self.v_cache_buffer:
             ctx.codebook_smoothing = True        # tokens generated later may quantize to symbols the prompt never produced
+            ctx.async_store = True               # appended blocks are encoded without waiting for the device
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, layer_idx: int,
                cache_kwargs: Optional[Dict[str, Any]] = None) -> Tuple[torch.Tensor, torch.Tensor]:

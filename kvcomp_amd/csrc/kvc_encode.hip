@@ -38,16 +38,69 @@ struct KvcEncodeArgs {
     uint16_t *thread_infos;
     uint8_t *encoded;
     int64_t encoded_cap;
-    uint32_t base_global_offset;
-    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload, [3] largest lane stream;
-                               // from word KVC_ENC_STATUS_WORDS on: payload bytes of tiles 1024 j .. 1024 j + 1023
-    uint32_t *idx_offset;      // {tiles, bytes}  (include/kernels.h:34-42)
+    uint32_t base_global_offset;   // what block_info.offset exceeds the position inside `encoded` by
+    uint32_t *status;          // [0] total payload bytes, [1] error bits, [2] largest tile payload, [3] largest lane stream,
+                               // [KVC_ENC_ST_BASE] block_info.offset of this call's first tile; from word
+                               // KVC_ENC_STATUS_WORDS on: payload bytes of tiles 1024 j .. 1024 j + 1023
+    uint32_t *idx_offset;      // {tiles, bytes}  (include/kernels.h:34-42); may be NULL
+    // several codebooks: table of tile row r = table + (r / rows_per_codebook) * table_stride (0: one table for all)
+    int64_t table_stride;
+    int rows_per_codebook;
+    const int32_t *codebook_meta;  // NULL, or int32[n_codebooks][4] from kvc_build_codebook_device (status in [3])
+    int n_codebooks;
+    // results left on the device (kvc_encode_async): see kvc_encode_job in include/kvcomp_hip.h
+    uint32_t *stream_bytes;    // NULL, or in / out: payload bytes already in `encoded`; this call appends behind them
+    uint32_t *result;          // NULL, or uint32[8]
 };
 
 constexpr int KVC_ENC_STATUS_WORDS = 16;            // status words in front of the per-1024-tile payload totals
+constexpr int KVC_ENC_ST_BASE = 5;
 constexpr uint32_t KVC_ENC_ERR_TILE_TOO_BIG = 1u;   // a tile payload exceeds 8191 bytes
 constexpr uint32_t KVC_ENC_ERR_NO_CODE = 2u;        // a symbol without a code (length 0 or outside the table)
 constexpr uint32_t KVC_ENC_ERR_CAPACITY = 4u;       // payload does not fit encoded_cap
+constexpr uint32_t KVC_ENC_ERR_CODEBOOK = 8u;       // a codebook was not built (status of kvc_build_codebook_device)
+
+// Table of the codebook that tile row `row` is encoded with.
+__device__ __forceinline__ const uint8_t *kvc_table_of_row(const KvcEncodeArgs &a, int64_t row)
+{
+    return a.rows_per_codebook ? a.table + (row / a.rows_per_codebook) * a.table_stride : a.table;
+}
+
+// First launch of an encode call: clears the status words (a kernel, not a memset, so that the call can be recorded
+// in a HIP graph), fixes the block_info.offset of the first tile (from the device counter when there is one) and
+// checks that every codebook was built.
+__global__ void __launch_bounds__(KVC_WAVE) kvc_encode_init_kernel(KvcEncodeArgs a)
+{
+    __shared__ uint32_t s_bad;
+    const int tid = threadIdx.x;
+    if (tid == 0) s_bad = 0;
+    __syncthreads();
+    if (a.codebook_meta)
+        for (int i = tid; i < a.n_codebooks; i += KVC_WAVE)
+            if (a.codebook_meta[4 * i + 3] != 0) atomicOr(&s_bad, KVC_ENC_ERR_CODEBOOK);
+    __syncthreads();
+    if (tid < KVC_ENC_STATUS_WORDS) {
+        uint32_t v = 0;
+        if (tid == 1) v = s_bad;
+        if (tid == KVC_ENC_ST_BASE) v = a.base_global_offset + (a.stream_bytes ? *a.stream_bytes : 0u);
+        a.status[tid] = v;
+    }
+}
+
+// Last launch: hands the call's outcome to the caller's device words (see kvc_encode_job).
+__global__ void kvc_encode_publish_kernel(KvcEncodeArgs a)
+{
+    const uint32_t total = a.status[0], err = a.status[1];
+    if (a.result) {
+        a.result[0] = total;
+        a.result[1] |= err;
+        if (a.status[2] > a.result[2]) a.result[2] = a.status[2];
+        if (a.status[3] > a.result[3]) a.result[3] = a.status[3];
+        a.result[4] += (uint32_t)a.tiles;
+        a.result[5] = a.status[KVC_ENC_ST_BASE];
+    }
+    if (a.stream_bytes && !err) *a.stream_bytes = a.status[KVC_ENC_ST_BASE] - a.base_global_offset + total;
+}
 
 // The 128 (or fewer) symbols of this lane's vector, 4 per register in stream order.
 //   K: token 64*row + lane, channels vec_len*col ..          (kernels.cu:439-444: one contiguous run)
@@ -108,26 +161,33 @@ __device__ __forceinline__ uint32_t kvc_count_tile(const KvcEncodeArgs &a, int64
     return longest;
 }
 
-__device__ __forceinline__ void kvc_load_len_table(const KvcEncodeArgs &a, uint8_t *s_len, int tid)
+// Code lengths of the table that `tile` is encoded with, one copy per wave (the tiles of a workgroup may lie in
+// rows with different codebooks).
+__device__ __forceinline__ void kvc_load_len_table(const KvcEncodeArgs &a, int64_t tile, uint8_t *s_len, int lane)
 {
-    uint32_t len = 0;
-    if (tid < a.table_entries) len = reinterpret_cast<const uint32_t *>(a.table)[2 * tid + 1];
-    s_len[tid] = (uint8_t)(len > 32 ? 0 : len);
+    const uint32_t *t = reinterpret_cast<const uint32_t *>(kvc_table_of_row(a, tile / a.cols));
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int i = lane + KVC_WAVE * k;
+        uint32_t len = 0;
+        if (i < a.table_entries) len = t[2 * i + 1];
+        s_len[i] = (uint8_t)(len > 32 ? 0 : len);
+    }
 }
 
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_count_kernel(KvcEncodeArgs a)
 {
-    __shared__ uint8_t s_len[256];
+    __shared__ uint8_t s_len[KVC_WAVES_PER_WG][256];
     __shared__ uint32_t s_err, s_longest;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) { s_err = 0; s_longest = 0; }
-    kvc_load_len_table(a, s_len, tid);
-    __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    if (tile < a.tiles) kvc_load_len_table(a, tile, s_len[wave], lane);
+    __syncthreads();
     if (tile < a.tiles) {
         uint32_t v[32];
         kvc_load_vector(a, tile, lane, v);
-        const uint32_t longest = kvc_count_tile(a, tile, lane, v, s_len, &s_err);
+        const uint32_t longest = kvc_count_tile(a, tile, lane, v, s_len[wave], &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
     }
     __syncthreads();
@@ -183,7 +243,7 @@ __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
     }
     if (lane == 0 && mx) atomicMax(&a.status[2], mx);
     __syncthreads();
-    uint32_t before = a.base_global_offset;
+    uint32_t before = a.status[KVC_ENC_ST_BASE];
     for (int w = 0; w < 16; w++) {
         before += s_before[w];
         if (w < wave) before += s_wave[w];
@@ -199,9 +259,12 @@ __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
             uint32_t total = 0;
             for (int w = 0; w < 16; w++) total += s_before[w];
             a.status[0] = total;
-            if ((int64_t)total > a.encoded_cap) atomicOr(&a.status[1], KVC_ENC_ERR_CAPACITY);
-            a.idx_offset[0] = (uint32_t)a.tiles;
-            a.idx_offset[1] = total;
+            const int64_t first = (int64_t)a.status[KVC_ENC_ST_BASE] - a.base_global_offset;      // position inside `encoded`
+            if (first + total > a.encoded_cap) atomicOr(&a.status[1], KVC_ENC_ERR_CAPACITY);
+            if (a.idx_offset) {
+                a.idx_offset[0] = (uint32_t)a.tiles;
+                a.idx_offset[1] = total;
+            }
         }
     }
 }
@@ -236,16 +299,21 @@ __device__ __forceinline__ KvcEmitPlace kvc_emit_place(const KvcEncodeArgs &a, i
     return p;
 }
 
-// The workgroup's copy of the encode table: entries without a usable code become {0, 0} (the count pass has
+// A wave's copy of the encode table of its tile: entries without a usable code become {0, 0} (the count pass has
 // flagged them), and *s_short tells whether every code has at most 8 bits (four then fit one 32-bit group).
-// The caller initialises *s_short to 1 and synchronises before and after.
-__device__ __forceinline__ void kvc_load_code_table(const KvcEncodeArgs &a, uint2 *s_table, uint32_t *s_short, int tid)
+// The caller initialises *s_short (the wave's own word) to 1 and synchronises before and after.
+__device__ __forceinline__ void kvc_load_code_table(const KvcEncodeArgs &a, int64_t tile, uint2 *s_table, uint32_t *s_short, int lane)
 {
-    uint2 e = tid < a.table_entries ? reinterpret_cast<const uint2 *>(a.table)[tid] : make_uint2(0u, 0u);
-    if (e.y > 32u) e = make_uint2(0u, 0u);
-    if (e.y < 32u) e.x &= (1u << e.y) - 1u;               // nothing above the code's own bits
-    s_table[tid] = e;
-    if (e.y > 8u) atomicAnd(s_short, 0u);
+    const uint2 *t = reinterpret_cast<const uint2 *>(kvc_table_of_row(a, tile / a.cols));
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int i = lane + KVC_WAVE * k;
+        uint2 e = i < a.table_entries ? t[i] : make_uint2(0u, 0u);
+        if (e.y > 32u) e = make_uint2(0u, 0u);
+        if (e.y < 32u) e.x &= (1u << e.y) - 1u;           // nothing above the code's own bits
+        s_table[i] = e;
+        if (e.y > 8u) atomicAnd(s_short, 0u);
+    }
 }
 
 // Pack this lane's vector MSB-first at its final position inside the (zeroed) LDS image of the tile payload.
@@ -315,16 +383,16 @@ __device__ __forceinline__ void kvc_write_image(const KvcEncodeArgs &a, const Kv
 
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a)
 {
-    __shared__ uint2 s_table[256];
-    __shared__ uint32_t s_short;
+    __shared__ uint2 s_table[KVC_WAVES_PER_WG][256];
+    __shared__ uint32_t s_short[KVC_WAVES_PER_WG];
     __shared__ uint32_t s_image[KVC_WAVES_PER_WG][KVC_IMAGE_WORDS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) s_short = 1u;
+    const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    if (lane == 0) s_short[wave] = 1u;
     __syncthreads();
-    kvc_load_code_table(a, s_table, &s_short, tid);
+    if (tile < a.tiles) kvc_load_code_table(a, tile, s_table[wave], &s_short[wave], lane);
     uint32_t *image = s_image[wave];
     __syncthreads();
-    const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
     const KvcEmitPlace p = kvc_emit_place(a, tile, tile < a.tiles);
     if (!p.ok) return;                                 // wave-uniform; each wave has its own image from here on
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
@@ -332,7 +400,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a
     uint32_t v[32];
     kvc_load_vector(a, tile, lane, v);
     kvc_wave_lds_sync();
-    kvc_pack_vector(a, tile, lane, v, s_table, image, p.head, s_short != 0u);
+    kvc_pack_vector(a, tile, lane, v, s_table[wave], image, p.head, s_short[wave] != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a, p, lane, image);
 }
@@ -487,20 +555,20 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
 template <bool IS_K>
 __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
 {
-    __shared__ uint8_t s_len[256];
+    __shared__ uint8_t s_len[KVC_WAVES_PER_WG][256];
     __shared__ uint32_t s_err, s_longest;
     __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];
     __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];   // V: {scale, 1 / scale, min, -} per token
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) { s_err = 0; s_longest = 0; }
-    kvc_load_len_table(a.e, s_len, tid);
-    __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    if (tile < a.e.tiles) kvc_load_len_table(a.e, tile, s_len[wave], lane);
+    __syncthreads();
     if (tile < a.e.tiles) {
         uint32_t v[32];
         if (IS_K) kvc_front_k<true>(a, tile, lane, s_sym[wave], v);
         else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
-        const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len, &s_err);
+        const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len[wave], &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
     }
     __syncthreads();
@@ -511,16 +579,16 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
 template <bool IS_K>
 __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
 {
-    __shared__ uint2 s_table[256];
+    __shared__ uint2 s_table[KVC_WAVES_PER_WG][256];
     __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];   // symbols first, then the payload image
     __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];
-    __shared__ uint32_t s_short;
+    __shared__ uint32_t s_short[KVC_WAVES_PER_WG];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    if (tid == 0) s_short = 1u;
-    __syncthreads();
-    kvc_load_code_table(a.e, s_table, &s_short, tid);
-    __syncthreads();
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
+    if (lane == 0) s_short[wave] = 1u;
+    __syncthreads();
+    if (tile < a.e.tiles) kvc_load_code_table(a.e, tile, s_table[wave], &s_short[wave], lane);
+    __syncthreads();
     const KvcEmitPlace p = kvc_emit_place(a.e, tile, tile < a.e.tiles);
     if (!p.ok) return;                                 // wave-uniform; nothing below involves another wave
     uint32_t *image = reinterpret_cast<uint32_t *>(s_sym[wave]);
@@ -531,7 +599,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
     for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
     kvc_wave_lds_sync();
-    kvc_pack_vector(a.e, tile, lane, v, s_table, image, p.head, s_short != 0u);
+    kvc_pack_vector(a.e, tile, lane, v, s_table[wave], image, p.head, s_short[wave] != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a.e, p, lane, image);
 }
@@ -546,61 +614,94 @@ struct KvcStoreSource {
     void *scale_f16;
 };
 
-static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, int64_t stride,
-                              const uint8_t *d_encode_table, int64_t encode_table_bytes, uint8_t *d_block_infos,
-                              uint8_t *d_thread_infos, uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
-                              uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes,
-                              int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream_,
-                              const KvcStoreSource *src = nullptr)
+// Everything an encode call is made of; the classic entry points fill in what they have and leave the rest zero.
+struct KvcEncodeCall {
+    int is_k;
+    const uint8_t *d_sym;
+    int64_t tokens, stride, head_dim;
+    const uint8_t *d_tables;
+    int64_t table_bytes, table_stride, rows_per_codebook;
+    const int32_t *d_meta;
+    uint8_t *d_block_infos, *d_thread_infos, *d_idx_offset, *d_encoded;
+    int64_t encoded_cap;
+    uint32_t base_global_offset;
+    uint32_t *d_stream_bytes, *d_result;
+    const KvcStoreSource *src;
+};
+
+static int kvc_encode_errors(uint32_t bits, uint32_t total, int64_t encoded_cap)
 {
-    hipStream_t stream = (hipStream_t)stream_;
+    if (bits & KVC_ENC_ERR_CODEBOOK) return kvc_fail(-3, "a codebook of this call was not built (fewer than two symbols, or not representable)");
+    if (bits & KVC_ENC_ERR_NO_CODE) return kvc_fail(-3, "a symbol has no code in the encode table");
+    if (bits & KVC_ENC_ERR_TILE_TOO_BIG)
+        return kvc_fail(-3, "a tile encodes to more than %d bytes, which thread_info (u16) cannot address", KVC_MAX_TILE_BYTES);
+    if (bits & KVC_ENC_ERR_CAPACITY)
+        return kvc_fail(-3, "payload (%u bytes) does not fit the encoded_data buffer (%lld bytes)", total, (long long)encoded_cap);
+    return 0;
+}
+
+// Queue the launches of one encode call (init, count, per-1024-tile sums, offsets, emit, publish); waits for nothing.
+// *slot receives the call's status words on the device.
+static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_t stream)
+{
     int64_t sizes[4];
-    if (int rc = kvc_calculate_buffer_size(tokens, stride, is_k, 0, head_dim, sizes)) return rc;
-    *h_total_bytes = 0;
-    if (tokens == 0) return 0;
-    KVC_REQUIRE(head_dim % 8 == 0, "head_dim must be a multiple of 8");
-    KVC_REQUIRE(encode_table_bytes > 0 && encode_table_bytes % 8 == 0 && encode_table_bytes <= 256 * 8,
+    if (int rc = kvc_calculate_buffer_size(c.tokens, c.stride, c.is_k, 0, c.head_dim, sizes)) return rc;
+    KVC_REQUIRE(c.tokens > 0, "nothing to encode");
+    KVC_REQUIRE(c.head_dim % 8 == 0, "head_dim must be a multiple of 8");
+    KVC_REQUIRE(c.table_bytes > 0 && c.table_bytes % 8 == 0 && c.table_bytes <= 256 * 8,
                 "encode table must hold 1..256 entries of 8 bytes");
-    KVC_REQUIRE(((uintptr_t)d_encode_table & 7) == 0 && ((uintptr_t)d_block_infos & 3) == 0 &&
-                ((uintptr_t)d_thread_infos & 1) == 0 && ((uintptr_t)d_idx_offset & 3) == 0 && ((uintptr_t)d_sym & 3) == 0,
+    KVC_REQUIRE(((uintptr_t)c.d_tables & 7) == 0 && ((uintptr_t)c.d_block_infos & 3) == 0 &&
+                ((uintptr_t)c.d_thread_infos & 1) == 0 && ((uintptr_t)c.d_idx_offset & 3) == 0 && ((uintptr_t)c.d_sym & 3) == 0 &&
+                ((uintptr_t)c.d_stream_bytes & 3) == 0 && ((uintptr_t)c.d_result & 3) == 0,
                 "encode buffers are misaligned");
-    KVC_REQUIRE(src != nullptr || d_sym != nullptr, "symbol pointer is NULL");
-    KVC_REQUIRE(stride % 4 == 0, "stride must be a multiple of 4");
+    KVC_REQUIRE(c.src != nullptr || c.d_sym != nullptr, "symbol pointer is NULL");
+    KVC_REQUIRE(c.stride % 4 == 0, "stride must be a multiple of 4");
+    KVC_REQUIRE(c.rows_per_codebook >= 0 && (c.rows_per_codebook == 0 || (c.table_stride >= c.table_bytes && c.table_stride % 8 == 0)),
+                "tables of several codebooks must be a multiple of 8 bytes apart and not overlap");
     void *slot;
     if (int rc = kvc_workspace_slot(&slot)) return rc;
     KvcEncodeArgs a;
-    a.sym = d_sym;
-    a.stride = stride;
-    a.is_k = is_k;
-    a.vec_len = is_k ? (int)head_dim : KVC_V_TOKENS;
-    a.cols = (int)(is_k ? stride / head_dim : stride / KVC_V_VEC_PER_BLK);
+    a.sym = c.d_sym;
+    a.stride = c.stride;
+    a.is_k = c.is_k;
+    a.vec_len = c.is_k ? (int)c.head_dim : KVC_V_TOKENS;
+    a.cols = (int)(c.is_k ? c.stride / c.head_dim : c.stride / KVC_V_VEC_PER_BLK);
     a.tiles = sizes[0] / 8;
-    a.table = d_encode_table;
-    a.table_entries = (int)(encode_table_bytes / 8);
-    a.block_infos = d_block_infos;
-    a.thread_infos = reinterpret_cast<uint16_t *>(d_thread_infos);
-    a.encoded = d_encoded;
-    a.encoded_cap = encoded_cap;
-    a.base_global_offset = base_global_offset;
+    a.table = c.d_tables;
+    a.table_entries = (int)(c.table_bytes / 8);
+    a.table_stride = c.table_stride;
+    a.rows_per_codebook = (int)c.rows_per_codebook;
+    a.codebook_meta = c.d_meta;
+    const int64_t rows = a.tiles / a.cols;
+    a.n_codebooks = c.rows_per_codebook ? (int)((rows + c.rows_per_codebook - 1) / c.rows_per_codebook) : 1;
+    a.block_infos = c.d_block_infos;
+    a.thread_infos = reinterpret_cast<uint16_t *>(c.d_thread_infos);
+    a.encoded = c.d_encoded;
+    a.encoded_cap = c.encoded_cap;
+    a.base_global_offset = c.base_global_offset;
     a.status = reinterpret_cast<uint32_t *>(slot);
-    a.idx_offset = reinterpret_cast<uint32_t *>(d_idx_offset);
+    a.idx_offset = reinterpret_cast<uint32_t *>(c.d_idx_offset);
+    a.stream_bytes = c.d_stream_bytes;
+    a.result = c.d_result;
     const int64_t chunks = (a.tiles + 1023) / 1024;
     KVC_REQUIRE((KVC_ENC_STATUS_WORDS + chunks) * 4 <= (int64_t)KVC_WS_SLOT_BYTES, "too many tiles (%lld) for one encode call",
                 (long long)a.tiles);
-    KVC_HIP(hipMemsetAsync(slot, 0, (size_t)KVC_ENC_STATUS_WORDS * 4, stream));
     const unsigned wgs = (unsigned)((a.tiles + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
+    const KvcStoreSource *src = c.src;
+    const int is_k = c.is_k;
     KvcStoreArgs sa;
     if (src) {
         sa.e = a;
         sa.x = reinterpret_cast<const __half *>(src->x_f16);
         sa.B = (int)src->B;
         sa.H = (int)src->H;
-        sa.D = (int)head_dim;
+        sa.D = (int)c.head_dim;
         sa.mask = src->mask;
         sa.eb = src->eb;
         sa.min_i8 = src->min_i8;
         sa.scale_f16 = reinterpret_cast<__half *>(src->scale_f16);
     }
+    hipLaunchKernelGGL(kvc_encode_init_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
     if (!src) hipLaunchKernelGGL(kvc_encode_count_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     else if (is_k) hipLaunchKernelGGL(kvc_store_count_kernel<true>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
     else hipLaunchKernelGGL(kvc_store_count_kernel<false>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
@@ -609,15 +710,46 @@ static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, in
     if (!src) hipLaunchKernelGGL(kvc_encode_emit_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     else if (is_k) hipLaunchKernelGGL(kvc_store_emit_kernel<true>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
     else hipLaunchKernelGGL(kvc_store_emit_kernel<false>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
+    if (a.result || a.stream_bytes) hipLaunchKernelGGL(kvc_encode_publish_kernel, dim3(1), dim3(1), 0, stream, a);
     KVC_HIP(hipGetLastError());
+    *slot_out = slot;
+    return 0;
+}
+
+static int kvc_entropy_encode(int is_k, const uint8_t *d_sym, int64_t tokens, int64_t stride,
+                              const uint8_t *d_encode_table, int64_t encode_table_bytes, uint8_t *d_block_infos,
+                              uint8_t *d_thread_infos, uint8_t *d_idx_offset, uint8_t *d_encoded, int64_t encoded_cap,
+                              uint32_t base_global_offset, int64_t head_dim, int64_t *h_total_bytes,
+                              int64_t *h_max_tile_bytes, int64_t *h_max_stream_bytes, void *stream_,
+                              const KvcStoreSource *src = nullptr)
+{
+    hipStream_t stream = (hipStream_t)stream_;
+    *h_total_bytes = 0;
+    if (tokens == 0) {
+        int64_t sizes[4];
+        return kvc_calculate_buffer_size(tokens, stride, is_k, 0, head_dim, sizes);
+    }
+    KvcEncodeCall c = {};
+    c.is_k = is_k;
+    c.d_sym = d_sym;
+    c.tokens = tokens;
+    c.stride = stride;
+    c.head_dim = head_dim;
+    c.d_tables = d_encode_table;
+    c.table_bytes = encode_table_bytes;
+    c.d_block_infos = d_block_infos;
+    c.d_thread_infos = d_thread_infos;
+    c.d_idx_offset = d_idx_offset;
+    c.d_encoded = d_encoded;
+    c.encoded_cap = encoded_cap;
+    c.base_global_offset = base_global_offset;
+    c.src = src;
+    void *slot;
+    if (int rc = kvc_encode_launch(c, &slot, stream)) return rc;
     uint32_t h_status[4] = {0, 0, 0, 0};
     KVC_HIP(hipMemcpyAsync(h_status, slot, 16, hipMemcpyDeviceToHost, stream));
     KVC_HIP(hipStreamSynchronize(stream));   // the reference returns after cudaDeviceSynchronize (kernels.cu:957)
-    if (h_status[1] & KVC_ENC_ERR_NO_CODE) return kvc_fail(-3, "a symbol has no code in the encode table");
-    if (h_status[1] & KVC_ENC_ERR_TILE_TOO_BIG)
-        return kvc_fail(-3, "a tile encodes to more than %d bytes, which thread_info (u16) cannot address", KVC_MAX_TILE_BYTES);
-    if (h_status[1] & KVC_ENC_ERR_CAPACITY)
-        return kvc_fail(-3, "payload (%u bytes) does not fit the encoded_data buffer (%lld bytes)", h_status[0], (long long)encoded_cap);
+    if (int rc = kvc_encode_errors(h_status[1], h_status[0], encoded_cap)) return rc;
     *h_total_bytes = h_status[0];
     if (h_max_tile_bytes) *h_max_tile_bytes = h_status[2];
     if (h_max_stream_bytes) *h_max_stream_bytes = h_status[3];
@@ -688,4 +820,70 @@ extern "C" int kvc_store_fused(int is_k, const void *d_x_f16, int64_t tokens, in
     return kvc_entropy_encode(is_k, nullptr, tokens, stride, d_encode_table, encode_table_bytes, d_block_infos, d_thread_infos,
                               d_idx_offset, d_encoded, encoded_cap, base_global_offset, head_dim, h_total_bytes,
                               h_max_tile_bytes, h_max_stream_bytes, stream, &src);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// encode without a host round trip: many codebooks per call, results left on the device (no counterpart in the
+// reference, whose encoder copies its counters to the host and waits for the device on every call,
+// kvcomp_cuda_extension/src/kernels.cu:950-965)
+// ---------------------------------------------------------------------------------------------------
+extern "C" int kvc_encode_async(const kvc_encode_job *job, void *stream)
+{
+    KVC_REQUIRE(job != nullptr, "NULL argument");
+    KVC_REQUIRE(job->batch > 0 && job->heads > 0 && job->head_dim > 0 && job->tokens > 0, "empty geometry");
+    KVC_REQUIRE(job->d_result != nullptr || job->d_stream_bytes != nullptr, "the call would leave no result anywhere");
+    const int64_t stride = job->batch * job->heads * job->head_dim;
+    KVC_REQUIRE(job->tokens % (job->is_k ? KVC_K_VEC_PER_BLK : KVC_V_VEC_LEN) == 0, "token count must be whole tiles");
+    KvcEncodeCall c = {};
+    c.is_k = job->is_k;
+    c.d_sym = job->d_sym;
+    c.tokens = job->tokens;
+    c.stride = stride;
+    c.head_dim = job->head_dim;
+    c.d_tables = job->d_encode_tables;
+    c.table_bytes = job->encode_table_bytes;
+    c.table_stride = job->table_stride_bytes;
+    c.rows_per_codebook = job->rows_per_codebook;
+    c.d_meta = job->d_codebook_meta;
+    c.d_block_infos = job->d_block_infos;
+    c.d_thread_infos = job->d_thread_infos;
+    c.d_idx_offset = nullptr;
+    c.d_encoded = job->d_encoded;
+    c.encoded_cap = job->encoded_cap;
+    c.base_global_offset = job->base_global_offset;
+    c.d_stream_bytes = job->d_stream_bytes;
+    c.d_result = job->d_result;
+    KvcStoreSource src = {job->d_x_f16, job->batch, job->heads, job->quant_mask, job->eb, job->d_min_i8, job->d_scale_f16};
+    if (!job->d_sym) {
+        KVC_REQUIRE(kvc_store_fused_supported(job->is_k, job->quant_mask, job->batch, job->heads, job->head_dim),
+                    "fused store: unsupported layout (is_k %d, groups 0x%x, %lld heads x %lld)", job->is_k, job->quant_mask,
+                    (long long)job->heads, (long long)job->head_dim);
+        KVC_REQUIRE(job->d_x_f16 != nullptr && job->d_min_i8 != nullptr && job->d_scale_f16 != nullptr, "NULL argument");
+        KVC_REQUIRE(((uintptr_t)job->d_x_f16 & 3) == 0 && ((uintptr_t)job->d_scale_f16 & 1) == 0, "fp16 buffers are misaligned");
+        KVC_REQUIRE(job->eb > 0.f, "error bound must be positive");
+        if (job->quant_mask != KVC_MASK_CHANNEL) {
+            const int64_t bs = KVC_K_VEC_PER_BLK;
+            if (int rc = kvc_quant_params(job->d_x_f16, job->tokens / bs, bs, job->batch, job->heads, job->head_dim, job->quant_mask,
+                                          job->eb, job->d_min_i8, job->d_scale_f16, stream))
+                return rc;
+        }
+        c.src = &src;
+    }
+    void *slot;
+    return kvc_encode_launch(c, &slot, (hipStream_t)stream);
+}
+
+extern "C" int kvc_encode_result(const uint32_t *d_result, int64_t encoded_cap, int64_t *h_total_bytes, int64_t *h_max_tile_bytes,
+                                 int64_t *h_max_stream_bytes, int64_t *h_tiles, void *stream)
+{
+    KVC_REQUIRE(d_result != nullptr, "NULL argument");
+    uint32_t h[8] = {};
+    KVC_HIP(hipMemcpyAsync(h, d_result, sizeof(h), hipMemcpyDeviceToHost, (hipStream_t)stream));
+    KVC_HIP(hipStreamSynchronize((hipStream_t)stream));
+    if (int rc = kvc_encode_errors(h[1], h[0], encoded_cap)) return rc;
+    if (h_total_bytes) *h_total_bytes = h[0];
+    if (h_max_tile_bytes) *h_max_tile_bytes = h[2];
+    if (h_max_stream_bytes) *h_max_stream_bytes = h[3];
+    if (h_tiles) *h_tiles = h[4];
+    return 0;
 }

@@ -122,6 +122,25 @@ class _Growable:
         self.data[self.used:self.used + n] = t
         self.used += n
 
+    def reserve(self, n: int, tail_shape, dtype, device):
+        """Make room for n more rows behind the filled part (which is kept); returns the view of those rows."""
+        if self.data is None:
+            self.data = torch.empty((n + max(n // 4, 16),) + tuple(tail_shape), dtype=dtype, device=device)
+        elif self.used + n > self.data.shape[0]:
+            cap = self.used + n + max((self.used + n) // 4, 16)
+            grown = torch.empty((cap,) + tuple(self.data.shape[1:]), dtype=self.data.dtype, device=self.data.device)
+            grown[:self.used] = self.data[:self.used]
+            self.data = grown
+        return self.data[self.used:self.used + n]
+
+    def trim(self):
+        """Give back what was reserved beyond a quarter of the filled part (after a worst-case reservation)."""
+        cap = self.used + max(self.used // 4, 16)
+        if self.data is not None and self.data.shape[0] > cap:
+            kept = torch.empty((cap,) + tuple(self.data.shape[1:]), dtype=self.data.dtype, device=self.data.device)
+            kept[:self.used] = self.data[:self.used]
+            self.data = kept
+
     @property
     def view(self) -> Optional[torch.Tensor]:
         return None if self.data is None else self.data[:self.used]
@@ -175,6 +194,46 @@ class KVCompCtx:
         self.max_stream_bytes = 0          # longest lane stream seen so far (sizes the fused decoders' LDS rows)
         self.encode_codebook: Optional[torch.Tensor] = None
         self.decode_codebook: Optional[torch.Tensor] = None
+        # what encodes that nobody waited for have left on the device: words 0 - 7 are kvc_encode_async's result words,
+        # word 8 counts the payload bytes in _encoded; _enc_pending bounds the bytes the host has not learnt of yet
+        self._state: Optional[torch.Tensor] = None
+        self._enc_pending = 0
+
+    def _device_state(self) -> torch.Tensor:
+        if self._state is None:
+            self._state = torch.zeros(16, dtype=torch.int32, device=self.device)
+            self._state[8] = self._encoded.used
+        return self._state
+
+    def _sync_sizes(self):
+        """Learn from the device how many payload bytes the encodes queued so far have produced (waits for them);
+        raises if one of them failed."""
+        if self._enc_pending == 0:
+            return
+        self._enc_pending = 0
+        _, max_tile, max_stream, _ = kvcomp_cuda.encode_result(self._state[:8], self._encoded.data.numel())
+        self._encoded.used = int(self._state[8].item())
+        self.max_tile_bytes = max(self.max_tile_bytes, max_tile)
+        self.max_stream_bytes = max(self.max_stream_bytes, max_stream)
+
+    def encoded_nosync(self):
+        """(payload buffer, upper bound of the bytes in use) without waiting for queued encodes: for callers that
+        only need an address and a bound, like the fused kernels."""
+        if self._encoded.data is None:
+            return None, 0
+        return self._encoded.data, min(self._encoded.used + self._enc_pending, self._encoded.data.numel())
+
+    def _append_encoded(self, encoded_: torch.Tensor):
+        self._sync_sizes()
+        self._encoded.append(encoded_)
+        if self._state is not None:
+            self._state[8] = self._encoded.used
+
+    @property
+    def encoded_data(self) -> Optional[torch.Tensor]:
+        """The reference's attribute (kvcomp_encode.py:56): the payload so far (waits for queued encodes)."""
+        self._sync_sizes()
+        return self._encoded.view
 
     @property
     def buffer(self) -> Optional[torch.Tensor]:
@@ -202,7 +261,6 @@ class KVCompCtx:
         self._tail_len = rest
 
     # the reference's public tensor attributes (kvcomp_encode.py:56-61)
-    encoded_data = property(lambda self: self._encoded.view)
     block_infos = property(lambda self: self._block_infos.view)
     thread_infos = property(lambda self: self._thread_infos.view)
     quant_min_ints = property(lambda self: self._min_ints.view)
@@ -269,12 +327,20 @@ class KVCompCtx:
         """Quantize + encode whole blocks [n * block_size, B, H, D] and append the stream; returns the symbols on the
         two-step path.  State is only touched after the library calls have succeeded."""
         mask = dims_to_mask(self.quant_dims)
+        if (not want_symbols and KVCompCtx.fused_store and self.async_store and self.encode_codebook is not None
+                and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
+            self._encode_direct(to_compress.shape[0], cache=to_compress, mask=mask, tables=self.encode_codebook,
+                                table_bytes=self.encode_codebook.numel())
+            return None
         if (not want_symbols and KVCompCtx.fused_store and self.encode_codebook is not None
                 and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
             self._store_fused(to_compress, mask)
             return None
         blocked = to_compress.reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
         quant_ints, min_ints, quant_scale = quant(blocked, self.quant_dims, self.quant_scale_rel)
+        if self.encode_codebook is None and self.device_codebook:
+            self._first_chunk_on_device(quant_ints, min_ints, quant_scale)
+            return quant_ints
         sizes = kvcomp_cuda.calculate_buffer_size(quant_ints, self.is_k, self.head_num, self.head_dim)
         KVCompCtx.buffer_ctx_len[self.device] = to_compress.shape[0]
         bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
@@ -294,13 +360,80 @@ class KVCompCtx:
             self._set_codebook(*codebook)
         self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
         self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
-        self._encoded.append(encoded_)
+        self._append_encoded(encoded_)
         self._block_infos.append(block_infos_)
         self._thread_infos.append(vec_infos_)
         self._min_ints.append(min_ints)
         self._scales.append(quant_scale)
         self.compressed_ctx_len += quant_ints.shape[0] * quant_ints.shape[1]
         return quant_ints
+
+    # The first chunk's codebook is built on the device (histogram, Huffman code, tables: no 256 reads of single counts
+    # by the host and no wait before the encode is queued); False: by the host builder, as in the reference.
+    device_codebook = True
+    # With a codebook in place, store(want_symbols=False) queues the fused quantize + encode and returns without
+    # waiting for it: sizes and errors are learnt the next time something asks for them (encoded_data, get_cr, ...),
+    # and a store that fails on the device is only reported then -- with its metadata already appended.  The caches
+    # that models use switch it on, together with codebook_smoothing, which rules out symbols without a code.
+    async_store = False
+
+    def _encode_direct(self, T: int, *, tables, table_bytes, symbols=None, cache=None, mask=0, meta=None,
+                       min_ints=None, quant_scale=None):
+        """Queue one encode whose outputs go straight to their final places in this context's buffers; nothing waits.
+        Quantizes `cache` on the fly (fused store) or takes `symbols` with their min_ints / quant_scale."""
+        nb = T // self.block_size
+        B, H, D = self.batch_size, self.head_num, self.head_dim
+        sizes = kvcomp_cuda.buffer_sizes(T, B * H * D, self.is_k, H, D)
+        gshape = mask_keepdim_shape((nb, self.block_size, B, H, D), dims_to_mask(self.quant_dims))
+        state = self._device_state()
+        bi = self._block_infos.reserve(sizes[0], (), torch.uint8, self.device)
+        ti = self._thread_infos.reserve(sizes[1], (), torch.uint8, self.device)
+        mn = self._min_ints.reserve(nb, gshape[1:], torch.int8, self.device)
+        sc = self._scales.reserve(nb, gshape[1:], torch.float16, self.device)
+        worst = T * B * H * D                                  # the reference's pre-allocation: a byte per symbol
+        if (self._encoded.data is None or
+                self._encoded.used + self._enc_pending + worst > self._encoded.data.numel()):
+            self._sync_sizes()                                 # growing copies the filled part: it has to be known
+            self._encoded.reserve(worst, (), torch.uint8, self.device)
+        if cache is None:
+            mn.copy_(min_ints)
+            sc.copy_(quant_scale)
+        kvcomp_cuda.encode_async(self.is_k, batch=B, head_num=H, head_dim=D, tokens=T, encode_tables=tables,
+                                 table_bytes=table_bytes, block_infos=bi, thread_infos=ti, encoded=self._encoded.data,
+                                 symbols=symbols, cache=cache, quant_mask=mask, eb=self.quant_scale_rel, min_ints=mn, scales=sc,
+                                 codebook_meta=meta, stream_bytes=state[8:9], result=state[:8])
+        self._block_infos.used += sizes[0]
+        self._thread_infos.used += sizes[1]
+        self._min_ints.used += nb
+        self._scales.used += nb
+        self._enc_pending += worst
+        self.compressed_ctx_len += T
+
+    def _first_chunk_on_device(self, quant_ints, min_ints, quant_scale):
+        """Codebook of the first stored chunk (kvcomp_encode.py:99-103) and its encode, queued back to back on the
+        device: histogram -> Huffman code and tables (kvc_build_codebook_device) -> encode with the table where it lies.
+        The host then reads the sizes (one wait) and keeps the codebook in the reference's form."""
+        counts = kvcomp_cuda.symbol_counts_chunks(quant_ints.reshape(-1), 1)
+        if self.codebook_smoothing:
+            counts[0, :self._smoothed_symbols()] += 1
+        enc, trees, meta = kvcomp_cuda.build_codebook_device(counts)
+        T = quant_ints.shape[0] * quant_ints.shape[1]
+        before = (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len)
+        self._encode_direct(T, tables=enc, table_bytes=enc.shape[1], symbols=quant_ints, meta=meta, min_ints=min_ints,
+                            quant_scale=quant_scale)
+        try:
+            self._sync_sizes()
+        except Exception:
+            (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len) = before
+            self._state[1] = 0                                 # the error has been reported; the context is as it was
+            raise
+        self._encoded.trim()                                   # a byte per symbol was reserved; the stream is a fraction of it
+        shift, enc_bytes, dec_bytes, status = (int(v) for v in meta[0].cpu())
+        assert status == 0 and shift == 0, "shift must be 0"
+        self._set_codebook(enc[0, :enc_bytes].cpu(), trees[0, :dec_bytes].cpu())
+
+    def _smoothed_symbols(self) -> int:
+        return min(256, int(math.ceil(1.0 / self.quant_scale_rel)) + 3)      # symbols 0 .. ceil(1 / eb) + 2
 
     # The reference derives the one codebook of a stream from its first stored chunk alone, so a symbol that first
     # shows up later has no code (its encoder then emits nothing for it and the stream is corrupt; here the
@@ -309,7 +442,7 @@ class KVCompCtx:
     codebook_smoothing = False
 
     def _smoothed_codebook(self, quant_ints: torch.Tensor):
-        n_sym = min(256, int(math.ceil(1.0 / self.quant_scale_rel)) + 3)      # symbols 0 .. ceil(1 / eb) + 2
+        n_sym = self._smoothed_symbols()
         counts = kvcomp_cuda.symbol_counts([quant_ints])
         counts[:n_sym] += 1
         shift, enc, dec = kvcomp_cuda.build_codebook_from_counts(counts)
@@ -332,7 +465,7 @@ class KVCompCtx:
             idx_buf, payload_buf, self._encoded.used)
         self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
         self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
-        self._encoded.append(encoded_)
+        self._append_encoded(encoded_)
         self._block_infos.append(block_infos_)
         self._thread_infos.append(vec_infos_)
         self._min_ints.append(min_ints)

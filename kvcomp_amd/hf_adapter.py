@@ -58,6 +58,7 @@ class KVCompLayer(CacheLayerMixin):
         self.v_ctx = KVCompCtx(False, B, H, D, cfg.v_quant_scale_rel)
         # the codebook comes from the prompt's first blocks; later tokens may quantize to symbols not seen there
         self.k_ctx.codebook_smoothing = self.v_ctx.codebook_smoothing = True
+        self.k_ctx.async_store = self.v_ctx.async_store = True      # appended blocks are encoded without waiting for the device
         self.is_initialized = True
 
     def update(self, key_states: torch.Tensor, value_states: torch.Tensor, *args, **kwargs) -> Tuple[torch.Tensor, torch.Tensor]:

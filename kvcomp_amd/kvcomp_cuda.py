@@ -203,6 +203,75 @@ def store_fused(is_k: bool, cache: torch.Tensor, quant_mask: int, quant_scale_re
     return encoded_data[:total.value], block_infos[:sizes[0]], thread_infos[:sizes[1]]
 
 
+def encode_async(is_k: bool, *, batch: int, head_num: int, head_dim: int, tokens: int, encode_tables: torch.Tensor,
+                 table_bytes: int, block_infos: torch.Tensor, thread_infos: torch.Tensor, encoded: torch.Tensor,
+                 symbols: torch.Tensor = None, cache: torch.Tensor = None, quant_mask: int = 0, eb: float = 0.0,
+                 min_ints: torch.Tensor = None, scales: torch.Tensor = None, table_stride: int = 0, rows_per_codebook: int = 0,
+                 codebook_meta: torch.Tensor = None, base_global_offset: int = 0, stream_bytes: torch.Tensor = None,
+                 result: torch.Tensor = None):
+    """kvc_encode_async: queue one encode (from `symbols`, or quantizing `cache` on the fly into min_ints / scales) with
+    one table per `rows_per_codebook` tile rows, and return without waiting.  `result` (device int32[8], zeroed once)
+    and `stream_bytes` (device int32[1]: payload bytes already in `encoded`, moved on by the call) stay on the device;
+    encode_result() reads them.  The output tensors are written from their first element on."""
+    job = _lib.EncodeJob()
+    job.is_k, job.quant_mask, job.eb = int(is_k), int(quant_mask), float(eb)
+    _require((symbols is None) != (cache is None), "give either symbols or cache")
+    dev = (symbols if symbols is not None else cache).device
+    if symbols is not None:
+        _dev_u8(symbols, "symbols")
+        _require(symbols.is_contiguous() and symbols.numel() == tokens * batch * head_num * head_dim, "symbols: wrong size")
+        job.d_sym = symbols.data_ptr()
+    else:
+        _require(cache.is_cuda and cache.dtype == torch.float16 and cache.is_contiguous() and
+                 cache.numel() == tokens * batch * head_num * head_dim, "cache must be a contiguous device float16 tensor [T, B, H, D]")
+        groups = _lib.lib().kvc_quant_groups(tokens // 64, 64, batch, head_num, head_dim, quant_mask)
+        _require(min_ints is not None and min_ints.dtype == torch.int8 and min_ints.numel() >= groups and min_ints.is_cuda,
+                 "min_ints: int8 device tensor of the group count")
+        _require(scales is not None and scales.dtype == torch.float16 and scales.numel() >= groups and scales.is_cuda,
+                 "scales: fp16 device tensor of the group count")
+        job.d_x_f16, job.d_min_i8, job.d_scale_f16 = cache.data_ptr(), min_ints.data_ptr(), scales.data_ptr()
+    sizes = buffer_sizes(tokens, batch * head_num * head_dim, is_k, head_num, head_dim)
+    for t, n, need in ((encode_tables, "encode_tables", table_bytes), (block_infos, "block_infos", sizes[0]),
+                       (thread_infos, "thread_infos", sizes[1]), (encoded, "encoded", 0)):
+        _dev_u8(t, n)
+        _require(t.numel() >= need, n + " buffer too small")
+    job.tokens, job.batch, job.heads, job.head_dim = tokens, batch, head_num, head_dim
+    job.d_encode_tables, job.encode_table_bytes = encode_tables.data_ptr(), table_bytes
+    job.table_stride_bytes, job.rows_per_codebook = table_stride, rows_per_codebook
+    if rows_per_codebook:
+        rows = tokens // (K_VEC_PER_BLK if is_k else V_VEC_LEN)
+        n_books = -(-rows // rows_per_codebook)
+        _require(encode_tables.numel() >= (n_books - 1) * table_stride + table_bytes, "encode_tables holds too few tables")
+        if codebook_meta is not None:
+            _require(codebook_meta.is_cuda and codebook_meta.dtype == torch.int32 and codebook_meta.numel() >= 4 * n_books,
+                     "codebook_meta: device int32 [n, 4]")
+    if codebook_meta is not None:
+        job.d_codebook_meta = codebook_meta.data_ptr()
+    job.d_block_infos, job.d_thread_infos = block_infos.data_ptr(), thread_infos.data_ptr()
+    job.d_encoded, job.encoded_cap = encoded.data_ptr(), encoded.numel()
+    job.base_global_offset = int(base_global_offset) & 0xFFFFFFFF
+    for t, n in ((stream_bytes, "stream_bytes"), (result, "result")):
+        if t is not None:
+            _require(t.is_cuda and t.dtype == torch.int32 and t.is_contiguous(), n + ": device int32 tensor")
+    _require(result is None or result.numel() >= 8, "result: 8 words")
+    if stream_bytes is not None:
+        job.d_stream_bytes = stream_bytes.data_ptr()
+    if result is not None:
+        job.d_result = result.data_ptr()
+    with torch.cuda.device(dev):
+        check(_lib.lib().kvc_encode_async(C.byref(job), C.c_void_p(torch.cuda.current_stream(dev).cuda_stream)))
+
+
+def encode_result(result: torch.Tensor, encoded_cap: int):
+    """kvc_encode_result: wait for the stream, raise if any call sharing `result` failed, and return
+    (payload bytes of the latest call, largest tile payload, longest lane stream, tiles encoded so far)."""
+    total, max_tile, max_stream, tiles = C.c_int64(0), C.c_int64(0), C.c_int64(0), C.c_int64(0)
+    with torch.cuda.device(result.device):
+        check(_lib.lib().kvc_encode_result(_ptr(result), encoded_cap, C.byref(total), C.byref(max_tile), C.byref(max_stream),
+                                           C.byref(tiles), _stream(result)))
+    return total.value, max_tile.value, max_stream.value, tiles.value
+
+
 def k_entropy_encode_cuda_export(input, encode_code_book, block_infos, thread_infos, idx_offset, encoded_data,
                                  base_global_offset: int, head_num: int, head_dim: int):
     """src/kernels.cu:919-966.  Returns views (payload, block_infos, thread_infos) of the caller's scratch."""

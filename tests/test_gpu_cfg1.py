@@ -54,9 +54,8 @@ def test_per_block_codebooks_round_trip(is_k):
     ti = torch.zeros(sizes[1], dtype=torch.uint8, device=DEV)
     payload = torch.zeros(sizes[3], dtype=torch.uint8, device=DEV)
     idx = torch.zeros(8, dtype=torch.uint8, device=DEV)
-    trees, used, total_bits = [], 0, 0
+    trees, total_bits = [], 0
     bi_per, ti_per = sizes[0] // n_books, sizes[1] // n_books
-    enc_fn = m.k_entropy_encode_cuda_export if is_k else m.v_entropy_encode_cuda_export
     dec_fn = m.k_entropy_decode_cuda_export if is_k else m.v_entropy_decode_cuda_export
     for blk in range(NB):
         s_blk = sym_d[blk]
@@ -66,32 +65,46 @@ def test_per_block_codebooks_round_trip(is_k):
         assert book == ref_book, "codebook of block %d" % blk
         assert np.array_equal(bits.cpu().numpy(), O.py_bits(ref_sym[blk], ref_book)), "bitstream of block %d" % blk
         total_bits += bits.numel()
+    # ---- all codebooks and the whole encode in three launches on the stream, no host round trip in between:
+    # per-codebook histograms -> Huffman codes and tables on the device -> one encode call that gives every tile
+    # row its own table
+    counts = m.symbol_counts_chunks(sym_d, n_books)
+    enc_tabs, trees_d, meta = m.build_codebook_device(counts, m.TREE_I8)
+    result = torch.zeros(8, dtype=torch.int32, device=DEV)
+    m.encode_async(is_k, batch=B, head_num=H, head_dim=D, tokens=T, symbols=sym_d, encode_tables=enc_tabs,
+                   table_bytes=enc_tabs.shape[1], table_stride=enc_tabs.shape[1], rows_per_codebook=1, codebook_meta=meta,
+                   block_infos=bi, thread_infos=ti, encoded=payload, result=result)
+    used, max_tile, max_stream, tiles = m.encode_result(result, payload.numel())
+    assert tiles == sizes[0] // 8 and 0 < max_stream <= max_tile <= 8191
+    meta_h = meta.cpu().numpy()
+    assert (meta_h[:, 3] == 0).all() and (meta_h[:, 0] == 0).all()
+    # per codebook, against the oracle: the table, and this row's tiles encoded with it at the offset the rows
+    # before it ended at
+    pos = 0
     for book_i in range(n_books):
         rows = slice(book_i * rows_per_tile_row, (book_i + 1) * rows_per_tile_row)
-        s_rows = sym_d[rows].contiguous()
-        shift, enc_tab, tree = m.build_codebook([s_rows])
-        assert shift == 0
+        counts_h = np.bincount(ref_sym[rows].ravel(), minlength=256).astype(np.int64)
+        code, length = O.huffman_build(counts_h)
+        _, ref_tab = O.encode_table(code, length, counts_h)
+        assert np.array_equal(enc_tabs[book_i, :int(meta_h[book_i, 1])].cpu().numpy(), ref_tab)
+        assert not enc_tabs[book_i, int(meta_h[book_i, 1]):].any()
+        # the host builder gives the same bytes (one construction serves both)
+        shift, enc_tab, tree = m.build_codebook([sym_d[rows].contiguous()])
+        assert shift == 0 and np.array_equal(enc_tab.numpy(), ref_tab)
+        assert np.array_equal(trees_d[book_i, :int(meta_h[book_i, 2])].cpu().numpy(), tree.numpy())
         trees.append(tree)
-        # the kernel-path codebook is the same code (one construction serves both, >= 2 symbols)
-        counts = np.bincount(ref_sym[rows].ravel(), minlength=256).astype(np.int64)
-        code, length = O.huffman_build(counts)
-        _, ref_tab = O.encode_table(code, length, counts)
-        assert np.array_equal(enc_tab.numpy(), ref_tab)
-        scratch_bi = torch.zeros(bi_per, dtype=torch.uint8, device=DEV)
-        scratch_ti = torch.zeros(ti_per, dtype=torch.uint8, device=DEV)
-        scratch_pl = torch.zeros(s_rows.numel(), dtype=torch.uint8, device=DEV)
-        enc, b_, t_ = enc_fn(s_rows, enc_tab.to(DEV), scratch_bi, scratch_ti, idx, scratch_pl, used, H, D)
-        ref_payload, ref_bi, ref_ti = O.encode_tiles(ref_sym[rows], is_k, ref_tab, used, vec_len=D if is_k else 128)
-        assert np.array_equal(enc.cpu().numpy(), ref_payload) and np.array_equal(b_.cpu().numpy(), ref_bi)
-        assert np.array_equal(t_.cpu().numpy(), ref_ti)
-        payload[used:used + enc.numel()] = enc
-        bi[book_i * bi_per:(book_i + 1) * bi_per] = b_
-        ti[book_i * ti_per:(book_i + 1) * ti_per] = t_
-        used += enc.numel()
+        ref_payload, ref_bi, ref_ti = O.encode_tiles(ref_sym[rows], is_k, ref_tab, pos, vec_len=D if is_k else 128)
+        assert np.array_equal(payload[pos:pos + ref_payload.size].cpu().numpy(), ref_payload), "payload of codebook %d" % book_i
+        assert np.array_equal(bi[book_i * bi_per:(book_i + 1) * bi_per].cpu().numpy(), ref_bi)
+        assert np.array_equal(ti[book_i * ti_per:(book_i + 1) * ti_per].cpu().numpy(), ref_ti)
+        pos += ref_payload.size
         # ---- decode this row with its own tree, out of the shared payload buffer
+        s_rows = sym_d[rows].contiguous()
         out = torch.zeros_like(s_rows)
-        dec_fn(payload[:used], b_.clone(), t_.clone(), tree.to(DEV), out, H, D)
+        dec_fn(payload[:pos], bi[book_i * bi_per:(book_i + 1) * bi_per].clone(), ti[book_i * ti_per:(book_i + 1) * ti_per].clone(),
+               tree.to(DEV), out, H, D)
         assert torch.equal(out, s_rows), "round trip of codebook %d" % book_i
+    assert pos == used
     # entropy-coded size is within a byte per lane stream of the whole-tensor coder's bit count
     assert total_bits / 8 <= used <= total_bits / 8 + T * B * H * D / 128 + 64
 

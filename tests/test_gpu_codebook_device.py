@@ -129,16 +129,22 @@ def test_per_block_codebooks_without_a_host_round_trip():
     bi = torch.zeros(sizes[0], dtype=torch.uint8, device=DEV)
     ti = torch.zeros(sizes[1], dtype=torch.uint8, device=DEV)
     payload = torch.zeros(sizes[3], dtype=torch.uint8, device=DEV)
-    idx = torch.zeros(8, dtype=torch.uint8, device=DEV)
-    bi_per, ti_per, used = sizes[0] // NB, sizes[1] // NB, 0
-    for blk in range(NB):
-        s_blk = sym[blk:blk + 1].contiguous()
-        sb, st_, sp = (torch.zeros(n, dtype=torch.uint8, device=DEV) for n in (bi_per, ti_per, s_blk.numel()))
-        e, b_, t_ = m.k_entropy_encode_cuda_export(s_blk, enc[blk, :int(meta_h[blk, 1])].contiguous(), sb, st_, idx, sp, used, H, D)
-        payload[used:used + e.numel()] = e
-        bi[blk * bi_per:(blk + 1) * bi_per] = b_
-        ti[blk * ti_per:(blk + 1) * ti_per] = t_
-        used += e.numel()
+    # one call encodes all sixteen blocks, each tile row with the table of its own codebook, straight from the
+    # tables the device builder wrote (a codebook that was not built would flag the call on the device)
+    result = torch.zeros(8, dtype=torch.int32, device=DEV)
+    m.encode_async(True, batch=B, head_num=H, head_dim=D, tokens=T, symbols=sym, encode_tables=enc, table_bytes=enc.shape[1],
+                   table_stride=enc.shape[1], rows_per_codebook=1, codebook_meta=meta, block_infos=bi, thread_infos=ti,
+                   encoded=payload, result=result)
+    used = m.encode_result(result, payload.numel())[0]
+    pos = 0
+    for blk in range(NB):                                                          # per block, against the oracle's encoder
+        h = np.bincount(ref_sym[blk].ravel(), minlength=256).astype(np.int64)
+        code, length = O.huffman_build(h)
+        _, ref_tab = O.encode_table(code, length, h)
+        ref_payload, ref_bi, ref_ti = O.encode_tiles(ref_sym[blk:blk + 1], True, ref_tab, pos, vec_len=D)
+        assert np.array_equal(payload[pos:pos + ref_payload.size].cpu().numpy(), ref_payload)
+        pos += ref_payload.size
+    assert pos == used
     q = S.synth_q(B, H, D).to(DEV)
     scores = torch.zeros(B, H, T, dtype=torch.float32, device=DEV)
     enc_all = payload[:used]

@@ -121,3 +121,140 @@ def test_fused_store_per_token_and_batch_groups(B, H, D):
     assert np.array_equal(g_min.cpu().numpy(), mn.ravel())
     assert np.array_equal(g_ti.cpu().numpy(), ti) and np.array_equal(g_bi.cpu().numpy(), bi)
     assert np.array_equal(g_enc.cpu().numpy(), payload)
+
+
+def _pair_of_contexts(T0, extra, B, H, D, k_mode="ChannelQuant"):
+    """The same tokens stored into a context that waits for every encode and into one that does not."""
+    from kvcomp_amd.ctx import KVCompCacheConfig, KVCompCacheConfigStatic, KVCompCtx, QuantMode
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("synthetic", QuantMode(k_mode), QuantMode("TokenQuant"), 64, 128,
+                                                       64, 128, 0.1, 0.2)
+    out = []
+    for is_k in (True, False):
+        x = (S.synth_k if is_k else S.synth_v)(T0 + extra, B, H, D).to(DEV)
+        pair = []
+        for asynchronous in (False, True):
+            ctx = KVCompCtx(is_k, B, H, D, 0.1 if is_k else 0.2)
+            ctx.codebook_smoothing = True
+            ctx.async_store = asynchronous
+            ctx.store(x[:T0], want_symbols=False)
+            for i in range(T0, T0 + extra):
+                ctx.store(x[i:i + 1], want_symbols=False)
+            pair.append(ctx)
+        out.append(pair)
+    return out
+
+
+@pytest.mark.parametrize("k_mode", ["ChannelQuant", "BlockQuant"])
+def test_store_without_waiting_gives_the_same_stream(k_mode):
+    """async_store queues the fused quantize + encode of every block that leaves the tail, writes its outputs straight
+    to their final places and never asks the device for a size; the stream must equal the waiting path's byte for
+    byte (payload, metadata, quantization parameters, size hints), and attention over it must not need the sizes."""
+    from kvcomp_amd.attention import CompressedAttention
+    B, H, D = 2, 2, 128
+    (k_sync, k_async), (v_sync, v_async) = _pair_of_contexts(300, 400, B, H, D, k_mode)
+    q = S.synth_q(B, 2 * H, D).to(DEV)
+    assert k_async._enc_pending > 0 and v_async._enc_pending > 0           # nobody has asked for a size yet
+    out_async = CompressedAttention(k_async, v_async).attend(q)            # an address and a bound are enough
+    assert k_async._enc_pending > 0
+    out_sync = CompressedAttention(k_sync, v_sync).attend(q)
+    assert torch.equal(out_async, out_sync)
+    for a, b in ((k_sync, k_async), (v_sync, v_async)):
+        assert a.compressed_ctx_len == b.compressed_ctx_len > 300 and a.ctx_len == b.ctx_len == 700
+        for name in ("encoded_data", "block_infos", "thread_infos", "quant_min_ints", "quant_scales", "buffer"):
+            assert torch.equal(getattr(a, name), getattr(b, name)), name
+        assert b._enc_pending == 0                                          # reading encoded_data learnt the sizes
+        assert (a.max_tile_bytes, a.max_stream_bytes) == (b.max_tile_bytes, b.max_stream_bytes)
+        assert a.get_cr() == b.get_cr()
+        assert torch.equal(a.get()[0], b.get()[0])
+
+
+def test_append_and_attend_can_be_captured_in_a_graph():
+    """One decode step of a layer -- append a block of tokens to K and V (quantize + encode, outputs in place) and
+    attend over everything -- recorded in a HIP graph: the step allocates nothing, waits for nothing and records no
+    memset.  The graph first puts the two device counters back where they stood, so that every replay appends at the
+    same place; each replay (with eager work in between) must equal the eager step bit for bit."""
+    from kvcomp_amd.attention import CompressedAttention
+    from kvcomp_amd.ctx import KVCompCacheConfig, KVCompCacheConfigStatic, KVCompCtx, QuantMode
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("synthetic", QuantMode.ChannelQuant, QuantMode.TokenQuant, 64, 128,
+                                                       64, 128, 0.1, 0.2)
+    B, H, Hq, D, T0, NEW = 2, 2, 4, 128, 512, 128
+    k, v = S.synth_k(T0 + NEW, B, H, D).to(DEV), S.synth_v(T0 + NEW, B, H, D).to(DEV)
+    q = S.synth_q(B, Hq, D).to(DEV)
+
+    def fresh():
+        kc, vc = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+        for c, x in ((kc, k), (vc, v)):
+            c.codebook_smoothing = True
+            c.async_store = True
+            c.store(x[:T0], want_symbols=False)
+        return kc, vc
+
+    kc, vc = fresh()
+    att = CompressedAttention(kc, vc)
+    kc.store(k[T0:], want_symbols=False)
+    vc.store(v[T0:], want_symbols=False)
+    eager = att.attend(q).clone()
+    torch.cuda.synchronize()
+
+    kc, vc = fresh()
+    att = CompressedAttention(kc, vc)
+    out = torch.empty(B, Hq, D, dtype=torch.float32, device=DEV)
+    att.attend(q, out=out)                                   # decode tables and workspace exist before the capture
+    # one eager step makes every buffer as large as the step needs; then the host's view is put back
+    saved = [(c._device_state().clone(), c._encoded.used, c._block_infos.used, c._thread_infos.used, c._min_ints.used,
+              c._scales.used, c.compressed_ctx_len, c.ctx_len, c._tail_len, c._enc_pending) for c in (kc, vc)]
+    kc.store(k[T0:], want_symbols=False)
+    vc.store(v[T0:], want_symbols=False)
+    att.attend(q, out=out)
+    torch.cuda.synchronize()
+
+    def rewind():
+        for c, sv in zip((kc, vc), saved):
+            c._state.copy_(sv[0])
+            (c._encoded.used, c._block_infos.used, c._thread_infos.used, c._min_ints.used, c._scales.used,
+             c.compressed_ctx_len, c.ctx_len, c._tail_len, c._enc_pending) = sv[1:]
+
+    def step():
+        rewind()
+        kc.store(k[T0:], want_symbols=False)
+        vc.store(v[T0:], want_symbols=False)
+        att.attend(q, out=out)
+
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        step()
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            step()
+    torch.cuda.synchronize()
+    for i in range(3):
+        out.fill_(float("nan"))
+        scratch = torch.randn(1 << 20, device=DEV).sum()     # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), i
+    assert kc.encoded_data.numel() > 0 and float(scratch) == float(scratch)
+
+
+def test_unbuilt_codebook_flags_the_encode_on_the_device():
+    """A codebook that kvc_build_codebook_device could not build (a block with one symbol only) makes the batched
+    encode fail when its result is read, not silently produce a stream."""
+    import kvcomp_amd.kvcomp_cuda as m
+    from kvcomp_amd._lib import KvcompError
+    T, B, H, D = 128, 1, 2, 128
+    sym = torch.randint(0, 9, (2, 64, B, H, D), dtype=torch.uint8, device=DEV)
+    sym[1] = 3                                               # the second block holds a single symbol
+    counts = m.symbol_counts_chunks(sym, 2)
+    enc, trees, meta = m.build_codebook_device(counts)
+    assert meta[:, 3].tolist() == [0, 1]
+    sizes = m.calculate_buffer_size(sym, True, H, D)
+    bi, ti = (torch.zeros(n, dtype=torch.uint8, device=DEV) for n in sizes[:2])
+    payload = torch.zeros(sizes[3], dtype=torch.uint8, device=DEV)
+    result = torch.zeros(8, dtype=torch.int32, device=DEV)
+    m.encode_async(True, batch=B, head_num=H, head_dim=D, tokens=T, symbols=sym, encode_tables=enc, table_bytes=enc.shape[1],
+                   table_stride=enc.shape[1], rows_per_codebook=1, codebook_meta=meta, block_infos=bi, thread_infos=ti,
+                   encoded=payload, result=result)
+    with pytest.raises(KvcompError, match="codebook"):
+        m.encode_result(result, payload.numel())
