@@ -76,6 +76,9 @@ int kvc_abi_version(void);
  *   "fused_mfma":           -1 (default): the multiply-accumulate of the fused matvecs runs on the matrix cores
  *                           (v_mfma_f32_4x4x4_16b_f16) where that is the faster kernel (rounded mode, codes of at most
  *                           7 bits); 0 never; 1 wherever the matrix-core kernels apply.
+ *   "fused_builtin_dpp":     0 (default): the fp32-FMA kernels pick their operand out of a quad of lanes with a permute
+ *                           written as inline assembly on the multiply-add itself; 1: through the compiler's lane-
+ *                           permute intrinsic (same result bit for bit; a cross-check against toolchain changes).
  *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
  *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile

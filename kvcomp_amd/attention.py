@@ -17,7 +17,7 @@ import torch
 
 from . import _lib, kvcomp_cuda
 from ._lib import check
-from .compute import dims_to_mask
+from .compute import dims_to_mask, expected_groups
 from .ctx import KVCompCtx
 
 
@@ -115,6 +115,11 @@ class CompressedAttention:
             d.d_thread_infos, d.thread_infos_bytes = ctx.thread_infos.data_ptr(), ctx.thread_infos.numel()
             enc, enc_bytes = ctx.encoded_nosync()          # an address and a bound: no wait for queued encodes
             d.d_encoded, d.encoded_bytes = enc.data_ptr(), enc_bytes
+            # the kernels take the quantization parameters by pointer: they must cover every group of the stream
+            groups = expected_groups(ctx.compressed_ctx_len, ctx.block_size, ctx.batch_size, ctx.head_num, ctx.head_dim, ctx.quant_dims)
+            assert ctx.quant_min_ints.numel() == groups and ctx.quant_scales.numel() == groups, \
+                "the context holds %d minima and %d scales for %d quantization groups" % (
+                    ctx.quant_min_ints.numel(), ctx.quant_scales.numel(), groups)
             d.d_quant_min_ints, d.d_quant_scales_f16 = ctx.quant_min_ints.data_ptr(), ctx.quant_scales.data_ptr()
         d.rows_per_codebook = 0
         d.quant_mask = dims_to_mask(ctx.quant_dims)

@@ -192,3 +192,14 @@ def apply_rotary_pos_emb_single(t, cos, sin, position_ids=None, unsqueeze_dim=1)
     cos = cos.unsqueeze(unsqueeze_dim)
     sin = sin.unsqueeze(unsqueeze_dim)
     return (t * cos) + (rotate_half(t) * sin)
+
+
+def expected_groups(compressed_ctx_len: int, block_size: int, batch: int, heads: int, head_dim: int, quant_dims) -> int:
+    """Number of (min, scale) pairs of a stream: one per combination of the dimensions of [NB, BS, B, H, D] that the
+    quantizer does not reduce over (utils/compute.py:93-106)."""
+    shape5 = (compressed_ctx_len // block_size, block_size, batch, heads, head_dim)
+    n = 1
+    for i, extent in enumerate(shape5):
+        if i not in quant_dims:
+            n *= extent
+    return n

@@ -29,6 +29,7 @@ from typing import Optional
 import numpy as np
 import torch
 
+from .compute import expected_groups
 from .ctx import KVCompCacheConfigStatic, KVCompCtx
 
 MAGIC = b"KVCOMP1\n"
@@ -123,7 +124,56 @@ def parse_header(data: bytes) -> dict:
                 raise ContainerError("section %s lies outside the data" % sec["name"])
             if int(np.prod(sec["shape"])) * item != sec["nbytes"]:
                 raise ContainerError("section %s: shape %s does not match %d bytes" % (sec["name"], sec["shape"], sec["nbytes"]))
+    check_consistency(header)
     return header
+
+
+_SECTION_DTYPES = {"encode_codebook": "u8", "decode_codebook": "u8", "block_infos": "u8", "thread_infos": "u8",
+                   "quant_min_ints": "i8", "quant_scales": "f16", "encoded_data": "u8", "tail": "f16"}
+
+
+def check_consistency(header: dict):
+    """The sections must describe one stream of the header's geometry: the kernels take these arrays by pointer, without
+    sizes, so a truncated or mismatched array would be read out of bounds on the device."""
+    def fail(msg):
+        raise ContainerError("inconsistent container: " + msg)
+    try:
+        is_k = bool(header["is_k"])
+        B, H, D = int(header["batch_size"]), int(header["head_num"]), int(header["head_dim"])
+        bs, total, comp = int(header["block_size"]), int(header["ctx_len"]), int(header["compressed_ctx_len"])
+        dims = [int(d) for d in header["quant_dims"]]
+        secs = {sec["name"]: sec for sec in header["sections"]}
+    except (KeyError, TypeError, ValueError) as e:
+        raise ContainerError("incomplete header: %s" % e)
+    if B <= 0 or H <= 0 or D <= 0 or D > 128 or D % 8 or bs <= 0:
+        fail("geometry %d x %d x %d, block %d" % (B, H, D, bs))
+    tile_tokens = 64 if is_k else 128
+    if not 0 <= comp <= total or comp % tile_tokens or comp % bs:
+        fail("%d of %d tokens compressed is not a whole number of %d-token tiles and %d-token blocks" % (comp, total, tile_tokens, bs))
+    if not is_k and (B * H * D) % 64:
+        fail("V rows of %d elements do not split into 64-channel tiles" % (B * H * D))
+    for name, dt in _SECTION_DTYPES.items():
+        if name not in secs:
+            fail("section %s is missing" % name)
+        if secs[name]["dtype"] != dt:
+            fail("section %s has dtype %s, expected %s" % (name, secs[name]["dtype"], dt))
+    def numel(name):
+        sec = secs[name]
+        return int(np.prod(sec["shape"])) if sec["nbytes"] else 0
+    tiles = comp // tile_tokens * (B * H if is_k else B * H * D // 64)
+    if numel("block_infos") != tiles * 8:
+        fail("block_infos holds %d bytes, %d tiles need %d" % (numel("block_infos"), tiles, tiles * 8))
+    if numel("thread_infos") != tiles * 64 * 2:
+        fail("thread_infos holds %d bytes, %d tiles need %d" % (numel("thread_infos"), tiles, tiles * 128))
+    groups = expected_groups(comp, bs, B, H, D, dims) if comp else 0
+    for name in ("quant_min_ints", "quant_scales"):
+        if numel(name) != groups:
+            fail("%s holds %d values, the stream has %d quantization groups" % (name, numel(name), groups))
+    if comp and (not numel("encoded_data") or not numel("decode_codebook") or not numel("encode_codebook")):
+        fail("a compressed part without payload or codebook")
+    tail_shape = list(secs["tail"]["shape"]) if secs["tail"]["nbytes"] else [0, B, H, D]
+    if tail_shape != [total - comp, B, H, D]:
+        fail("the tail has shape %s, expected %s" % (tail_shape, [total - comp, B, H, D]))
 
 
 def loads(data: bytes, device: Optional[torch.device] = None) -> KVCompCtx:

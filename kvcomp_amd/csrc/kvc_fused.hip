@@ -100,16 +100,23 @@ __device__ __noinline__ KvcVec<REP> kvc_slow_tile(const uint32_t *words, uint32_
 // acc += x * (the value of `quad` in lane (l & ~3) + J of lane l's quad): the lane permute rides on the FMA's
 // first operand, so picking one of the four operands a quad holds costs no instruction of its own.
 // (`quad` comes straight from an LDS read and `acc` is not the permuted operand, so no VALU-write -> permuted-read
-// hazard can arise between consecutive FMAs.)
-template <int J>
+// hazard can arise between consecutive FMAs.)  The inline assembly is opaque to the compiler's hazard recogniser, so it
+// has a twin (BUILTIN) that expresses the same permute through the compiler's own intrinsic and leaves instruction
+// selection and hazard handling to it; KvcFusedArgs::builtin_dpp selects it, and a test holds the two to equal bits.
+template <int J, bool BUILTIN>
 __device__ __forceinline__ void kvc_fma_quad_pick(float &acc, uint32_t quad, float x)
 {
-    asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[%3,%3,%3,%3] row_mask:0xf bank_mask:0xf"
-        : "+v"(acc)
-        : "v"(quad), "v"(x), "n"(J));
+    if (BUILTIN) {
+        const int picked = __builtin_amdgcn_update_dpp(0, (int)quad, J * 0x55 /* quad_perm:[J,J,J,J] */, 0xf, 0xf, false);
+        acc = fmaf(__int_as_float(picked), x, acc);
+    } else {
+        asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[%3,%3,%3,%3] row_mask:0xf bank_mask:0xf"
+            : "+v"(acc)
+            : "v"(quad), "v"(x), "n"(J));
+    }
 }
 
-template <int G, bool CHECK, bool SKEW, int REP>
+template <int G, bool CHECK, bool SKEW, int REP, bool BUILTIN>
 __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t &u,
                                              uint32_t fentry_base, uint32_t mask4, int n,
                                              const float *ops, float (&acc)[REP], uint32_t &worst)
@@ -139,7 +146,7 @@ __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t &u,
             kvc_static_for<REP>([&](auto r_) {
                 constexpr int r = decltype(r_)::value;
                 constexpr int k = g * REP + r;
-                kvc_fma_quad_pick<k & 3>(acc[r], blk[k >> 2], f);
+                kvc_fma_quad_pick<k & 3, BUILTIN>(acc[r], blk[k >> 2], f);
             });
         });
         const uint32_t used = es & 0xffu;
@@ -151,7 +158,7 @@ __device__ __forceinline__ void kvc_fast_dot(const uint32_t *stage, uint32_t &u,
 // The same with 64 stream bits per refill from LDS: G symbols are decoded from the low word, the window is
 // re-formed from the register pair at the bits consumed so far (fewer than 32 unless the group overflowed, which
 // `worst` reports), G more follow.  Halves the refills (address arithmetic, LDS round trip, length sums) per symbol.
-template <int G, bool CHECK, bool SKEW, int REP>
+template <int G, bool CHECK, bool SKEW, int REP, bool BUILTIN>
 __device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t &u,
                                               uint32_t fentry_base, uint32_t mask4, int n,
                                               const float *ops, float (&acc)[REP], uint32_t &worst)
@@ -180,7 +187,7 @@ __device__ __forceinline__ void kvc_fast_dot2(const uint32_t *stage, uint32_t &u
             kvc_static_for<REP>([&](auto r_) {
                 constexpr int r = decltype(r_)::value;
                 constexpr int k = g * REP + r;
-                kvc_fma_quad_pick<k & 3>(acc[r], blk[k >> 2], f);
+                kvc_fma_quad_pick<k & 3, BUILTIN>(acc[r], blk[k >> 2], f);
             });
         });
         const uint32_t used = es & 0xffu;
@@ -233,7 +240,7 @@ __device__ __forceinline__ void kvc_rounded_dot(const uint32_t *stage, uint32_t 
 typedef uint32_t kvc_u32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) kvc_u32x2 kvc_lds_u32x2;
 
-template <bool SKEW, int REP>
+template <bool SKEW, int REP, bool BUILTIN>
 __device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t &u, uint32_t mask8,
                                              uint32_t table_base, int n, const float *ops, float (&acc)[REP])
 {
@@ -257,8 +264,8 @@ __device__ __forceinline__ void kvc_pair_dot(const uint32_t *stage, uint32_t &u,
             kvc_static_for<REP>([&](auto r_) {
                 constexpr int r = decltype(r_)::value;
                 constexpr int k0 = (2 * p) * REP + r, k1 = (2 * p + 1) * REP + r;
-                kvc_fma_quad_pick<k0 & 3>(acc[r], blk[k0 >> 2], __uint_as_float(e.x));
-                kvc_fma_quad_pick<k1 & 3>(acc[r], blk[k1 >> 2], __uint_as_float(e.y));
+                kvc_fma_quad_pick<k0 & 3, BUILTIN>(acc[r], blk[k0 >> 2], __uint_as_float(e.x));
+                kvc_fma_quad_pick<k1 & 3, BUILTIN>(acc[r], blk[k1 >> 2], __uint_as_float(e.y));
             });
         });
         u += es & 0xffu;
@@ -498,33 +505,38 @@ __global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_ke
             const uint32_t *words = a.row_words ? rows + lane * a.row_words : pack;
             const bool skew = !a.row_words && a.skew;
             uint32_t u = st.u0, worst = 0;
-            auto run = [&](auto skew_) {
-                constexpr bool SK = decltype(skew_)::value;
+            auto run = [&](auto skew_, auto builtin_) {
+                constexpr bool SK = decltype(skew_)::value, BI = decltype(builtin_)::value;
                 if (pairs) {
-                    kvc_pair_dot<SK, REP>(words, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
+                    kvc_pair_dot<SK, REP, BI>(words, u, ((1u << pbits) - 1u) << 3, fe, n, my_ops, acc);
                 } else if (dwin && !fcheck) {
-                    if (fgroup >= 8) kvc_fast_dot2<8, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
-                    else if (fgroup == 7) kvc_fast_dot2<7, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
-                    else if (fgroup == 6) kvc_fast_dot2<6, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
-                    else if (fgroup == 5) kvc_fast_dot2<5, false, SK, REP>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    if (fgroup >= 8) kvc_fast_dot2<8, false, SK, REP, BI>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 7) kvc_fast_dot2<7, false, SK, REP, BI>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 6) kvc_fast_dot2<6, false, SK, REP, BI>(words, u, fe, mask4, n_main, my_ops, acc, worst);
+                    else if (fgroup == 5) kvc_fast_dot2<5, false, SK, REP, BI>(words, u, fe, mask4, n_main, my_ops, acc, worst);
                     const int rest = fgroup == 4 ? n : n - n_main;
-                    if (rest) kvc_fast_dot2<4, false, SK, REP>(words, u, fe, mask4, rest, my_ops + (n - rest) * REP, acc, worst);
+                    if (rest) kvc_fast_dot2<4, false, SK, REP, BI>(words, u, fe, mask4, rest, my_ops + (n - rest) * REP, acc, worst);
                 } else if (dwin && fgroup >= 4 && fgroup < 8) {
-                    kvc_fast_dot2<4, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot2<4, true, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else if (fgroup >= 8 && !fcheck) {
-                    kvc_fast_dot<8, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot<8, false, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else if (fgroup >= 8) {
-                    kvc_fast_dot<8, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot<8, true, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else if (fgroup >= 4 && !fcheck) {
-                    kvc_fast_dot<4, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot<4, false, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else if (fgroup >= 4) {
-                    kvc_fast_dot<4, true, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot<4, true, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 } else {
-                    kvc_fast_dot<2, false, SK, REP>(words, u, fe, mask4, n, my_ops, acc, worst);
+                    kvc_fast_dot<2, false, SK, REP, BI>(words, u, fe, mask4, n, my_ops, acc, worst);
                 }
             };
-            if (skew) run(std::true_type{});
-            else run(std::false_type{});
+            if (a.builtin_dpp) {
+                if (skew) run(std::true_type{}, std::true_type{});
+                else run(std::false_type{}, std::true_type{});
+            } else {
+                if (skew) run(std::true_type{}, std::false_type{});
+                else run(std::false_type{}, std::false_type{});
+            }
             redo = __any(worst > 30u);
         }
         if (redo) {
@@ -844,6 +856,7 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     a.expand = 0;
     a.out_words = 0;
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
+    a.builtin_dpp = kvc_option(KVC_OPT_FUSED_BUILTIN_DPP) != 0;
     if (allow_pairs && extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
         a.pair_bits = 2 * max_code_bits;
         // eight bytes per entry (fp32 symbols), four in the matrix-core kernels (fp16 symbols)

@@ -31,6 +31,7 @@ struct KvcFusedArgs {
     int row_words;       // LDS words per lane stream (odd); 0 = decode from the packed payload
     int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
     int double_window;   // refill 64 stream bits at a time where the vector length allows
+    int builtin_dpp;     // fp32-FMA kernels: lane permutes through the compiler's intrinsic instead of inline assembly
     // kvc_expand_kernel (plain decode, decode + dequantize): no x; the operand table holds {scale, min} per element
     // Rounded mode of the matvec kernels: every (sym + min) * scale is rounded to fp16 before it meets q / p, as the
     // reference's dequantizer does (models/cache/kvcomp_encode.py:146); the operand table then holds

@@ -54,6 +54,7 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"fused_rounded", "KVCOMP_FUSED_ROUNDED", 1},                // 1: round each dequantized value to fp16 before the matvec, as the reference's dequantizer does
     {"attention_tail_in_merge", "KVCOMP_ATTENTION_TAIL_IN_MERGE", 1},   // kvc_attention_decode: V's fp16 tail inside the merge kernel
     {"fused_mfma", "KVCOMP_FUSED_MFMA", -1},                     // matrix-core kernels: -1 where they are faster (rounded mode), 0 never, 1 always
+    {"fused_builtin_dpp", "KVCOMP_FUSED_BUILTIN_DPP", 0},        // fp32-FMA kernels: the quad permute through the compiler's intrinsic, not inline assembly
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;

@@ -323,6 +323,10 @@ def decode_dequant(is_k: bool, in_tensor, block_infos, thread_infos, decode_code
              "out must be a contiguous device float16 tensor [T, B, H, D]")
     _require(quant_min_ints.dtype == torch.int8 and quant_scales.dtype == torch.float16, "min_ints int8, scales fp16")
     T, B, H, D = out.shape
+    # the kernel takes the quantization parameters by pointer: they must cover every group of the stream
+    groups = _lib.lib().kvc_quant_groups(T // block_size, block_size, B, H, D, quant_mask) if block_size > 0 and T % block_size == 0 else -1
+    _require(quant_min_ints.numel() == groups and quant_scales.numel() == groups,
+             "%d minima and %d scales for %d quantization groups" % (quant_min_ints.numel(), quant_scales.numel(), groups))
     ms = C.c_float(0.0)
     with torch.cuda.device(out.device):
         check(_lib.lib().kvc_decode_dequant(int(is_k), _ptr(in_tensor), in_tensor.numel(), _ptr(block_infos), block_infos.numel(),

@@ -44,6 +44,55 @@ def test_framing_alignment_and_validation():
             Cn.parse_header(bad)
 
 
+def _rewrite_header(blob, edit):
+    """The same container with its JSON header edited (the sections keep their places)."""
+    import json
+    (hlen,) = struct.unpack("<Q", blob[8:16])
+    header = json.loads(blob[16:16 + hlen].decode())
+    edit(header)
+    body = json.dumps(header).encode()
+    assert len(body) <= hlen
+    return blob[:16] + body + b" " * (hlen - len(body)) + blob[16 + hlen:]
+
+
+def test_inconsistent_sections_are_refused():
+    """The kernels take the arrays of a stream by pointer, so a container whose sections do not fit its header's
+    geometry (too few quantization parameters, a short tail, metadata of another tile count, a wrong dtype, a token
+    count that is not whole tiles) must be refused before any tensor reaches the device."""
+    from kvcomp_amd import container as Cn
+    blob = Cn.dumps(_Stub())
+    Cn.parse_header(blob)                                            # the undamaged container is fine
+
+    def section(h, name):
+        return next(s for s in h["sections"] if s["name"] == name)
+
+    def shrink(name, shape, itemsize):
+        def edit(h):
+            s = section(h, name)
+            s["shape"], s["nbytes"] = shape, int(np.prod(shape)) * itemsize
+        return edit
+
+    damaged = {
+        "too few scales": shrink("quant_scales", [1, 1, 1, 2, 4], 2),
+        "too few minima": shrink("quant_min_ints", [1, 1, 1, 1, 8], 1),
+        "short tail": shrink("tail", [5, 1, 2, 8], 2),
+        "tail of another head count": shrink("tail", [6, 1, 1, 8], 2),
+        "block_infos of one tile only": shrink("block_infos", [8], 1),
+        "thread_infos too short": shrink("thread_infos", [128], 1),
+        "scales stored as bytes": lambda h: section(h, "quant_scales").update(dtype="u8", nbytes=16),
+        "compressed part is not whole tiles": lambda h: h.update(compressed_ctx_len=60, ctx_len=66),
+        "more compressed than stored": lambda h: h.update(ctx_len=32),
+        "more heads than the sections cover": lambda h: h.update(head_num=4),
+        "head_dim the kernels do not take": lambda h: h.update(head_dim=12),
+        "section missing": lambda h: h["sections"].pop(3),
+        "no payload": lambda h: section(h, "encoded_data").update(nbytes=0, offset=0, shape=None),
+    }
+    for what, edit in damaged.items():
+        with pytest.raises(Cn.ContainerError):
+            Cn.parse_header(_rewrite_header(blob, edit))
+            pytest.fail("accepted: " + what)
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("D", [128, 96])
 def test_save_load_round_trip_on_gpu(tmp_path, D):

@@ -243,6 +243,41 @@ def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D, 
     assert L.kvc_set_option(b"no_such_option", 1) != 0
 
 
+@pytest.mark.parametrize("D,rep,eb_k", [(128, 1, 0.1), (96, 2, 0.05), (64, 4, 0.3), (128, 8, 0.1)])
+def test_lane_permute_in_assembly_equals_the_compilers(D, rep, eb_k):
+    """The fp32-FMA kernels fetch one of four operands from the lanes of a quad with a permute that rides on the
+    multiply-add (inline assembly, which the compiler's hazard handling cannot see into).  The same kernels with
+    the permute expressed through the compiler's intrinsic must give the same bits, for the one-symbol loops (K)
+    and the two-symbol loop (V), skewed and plain staging, one and two tiles per wave."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant", ebk=eb_k)
+    T, B, H = 1024 + 13, 2, 2
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, eb_k), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    saved = {n: _lib.set_option(n, v_) for n, v_ in (("fused_rounded", 0), ("fused_mfma", 0))}
+    try:
+        for skew in (0, 1):
+            for tpw in (1, 2):
+                _lib.set_option("fused_skew", skew)
+                _lib.set_option("fused_tiles_per_wave", tpw)
+                _lib.set_option("fused_builtin_dpp", 0)
+                asm = CompressedAttention(kctx, vctx).attend(q)
+                _lib.set_option("fused_builtin_dpp", 1)
+                builtin = CompressedAttention(kctx, vctx).attend(q)
+                assert torch.isfinite(asm).all() and torch.equal(asm, builtin), (skew, tpw)
+    finally:
+        for n, v_ in saved.items():
+            _lib.set_option(n, v_)
+        _lib.set_option("fused_skew", -1)
+        _lib.set_option("fused_tiles_per_wave", 0)
+        _lib.set_option("fused_builtin_dpp", 0)
+
+
 @pytest.mark.parametrize("hint", ["too_small", "absent"])
 def test_compressed_attention_with_wrong_or_missing_size_hints(hint, fused_mode):
     """The encoder's size hints only size the LDS staging: with hints that are too small (tiles do not fit and
