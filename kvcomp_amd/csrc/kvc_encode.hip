@@ -125,9 +125,17 @@ __device__ __forceinline__ void kvc_load_vector(const KvcEncodeArgs &a, int64_t 
     }
 }
 
-// Count pass for one tile: thread_infos, byte_num, error bits; returns the lane-stream maximum of the wave.
-__device__ __forceinline__ uint32_t kvc_count_tile(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
-                                                   const uint8_t *s_len, uint32_t *s_err)
+// What the count step of one tile finds out (every field wave-uniform except `start`).
+struct KvcTileCount {
+    uint32_t start;      // first byte of this lane's stream inside the tile payload
+    uint32_t bytes;      // payload bytes of the tile
+    uint32_t longest;    // longest lane stream of the tile
+    uint32_t err;        // error bits raised by any lane
+};
+
+// Count step for one tile: adds up the code lengths of the lane's vector, writes the 64 thread_infos.
+__device__ __forceinline__ KvcTileCount kvc_count_vectors(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
+                                                          const uint8_t *s_len)
 {
     uint32_t bits = 0, bad = 0;
     const int nd = a.vec_len >> 2;
@@ -145,20 +153,30 @@ __device__ __forceinline__ uint32_t kvc_count_tile(const KvcEncodeArgs &a, int64
     const uint32_t bytes = (bits + 7u) >> 3;
     const uint32_t end = kvc_wave_inclusive_scan(bytes, lane);
     a.thread_infos[tile * KVC_WAVE + lane] = (uint16_t)((end << 3) + (bytes << 3) - bits);
-    uint32_t err = bad ? KVC_ENC_ERR_NO_CODE : 0u;
-    if (lane == KVC_WAVE - 1) {
-        if (end > (uint32_t)KVC_MAX_TILE_BYTES) err |= KVC_ENC_ERR_TILE_TOO_BIG;
-        // byte_num; the offset half of block_info is filled in by the scan kernel
-        reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[1] = end > 0xffffu ? 0xffffu : end;
-    }
-    if (err) atomicOr(s_err, err);
+    KvcTileCount c;
+    c.start = end - bytes;
+    c.bytes = (uint32_t)__builtin_amdgcn_readlane((int)end, KVC_WAVE - 1);
+    c.err = __any(bad) ? KVC_ENC_ERR_NO_CODE : 0u;
+    if (c.bytes > (uint32_t)KVC_MAX_TILE_BYTES) c.err |= KVC_ENC_ERR_TILE_TOO_BIG;
     uint32_t longest = bytes;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         const uint32_t o = (uint32_t)__shfl_xor((int)longest, off, 64);
         longest = o > longest ? o : longest;
     }
-    return longest;
+    c.longest = longest;
+    return c;
+}
+
+// Count pass for one tile: thread_infos, byte_num, error bits; returns the lane-stream maximum of the wave.
+__device__ __forceinline__ uint32_t kvc_count_tile(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
+                                                   const uint8_t *s_len, uint32_t *s_err)
+{
+    const KvcTileCount c = kvc_count_vectors(a, tile, lane, v, s_len);
+    // byte_num; the offset half of block_info is filled in by the scan kernel
+    if (lane == KVC_WAVE - 1) reinterpret_cast<uint32_t *>(a.block_infos + 8 * tile)[1] = c.bytes > 0xffffu ? 0xffffu : c.bytes;
+    if (c.err && lane == 0) atomicOr(s_err, c.err);
+    return c.longest;
 }
 
 // Code lengths of the table that `tile` is encoded with, one copy per wave (the tiles of a workgroup may lie in
@@ -321,10 +339,15 @@ __device__ __forceinline__ void kvc_load_code_table(const KvcEncodeArgs &a, int6
 // image (what is left above the live bits is never read again, so it is not cleared).  With codes of at most
 // 8 bits the four symbols of a register are first joined into one group of at most 32 bits, which costs a
 // quarter of the accumulator traffic.
-__device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, int64_t tile, int lane, const uint32_t (&v)[32],
+// Where lane `lane`'s stream starts inside the payload of `tile`, from the thread_infos an earlier launch wrote.
+__device__ __forceinline__ uint32_t kvc_stream_start(const KvcEncodeArgs &a, int64_t tile, int lane)
+{
+    return lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
+}
+
+__device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, uint32_t start, const uint32_t (&v)[32],
                                                 const uint2 *s_table, uint32_t *image, uint32_t head, bool short_codes)
 {
-    const uint32_t start = lane ? (uint32_t)(a.thread_infos[tile * KVC_WAVE + lane - 1] >> 3) : 0u;
     const uint32_t bitpos = (head + start) * 8u;
     uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
     uint64_t acc = 0;
@@ -400,7 +423,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a
     uint32_t v[32];
     kvc_load_vector(a, tile, lane, v);
     kvc_wave_lds_sync();
-    kvc_pack_vector(a, tile, lane, v, s_table[wave], image, p.head, s_short[wave] != 0u);
+    kvc_pack_vector(a, kvc_stream_start(a, tile, lane), v, s_table[wave], image, p.head, s_short[wave] != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a, p, lane, image);
 }
@@ -497,6 +520,61 @@ __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile,
     for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
 }
 
+// The count pass's variant: the lane keeps its two channels of all 64 tokens in registers (64 loads in flight, one walk
+// over the tile instead of two), finds the groups' minima and maxima there, publishes the group parameters and quantizes.
+__device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t (&v)[32])
+{
+    const int64_t stride = a.e.stride;
+    const int D = a.D, RS = D + 4;
+    const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
+    const bool act = 2 * lane < D;
+    const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (act ? 2 * lane : 0);
+    auto lo = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); };
+    auto hi = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); };
+    uint32_t raw[KVC_WAVE];
+#pragma unroll
+    for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + t * stride);
+    KvcGroupParams g0, g1;
+    if (a.mask == KVC_MASK_CHANNEL) {
+        const int64_t g = row * stride + col * D + (act ? 2 * lane : 0);
+        float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+#pragma unroll
+        for (int t = 0; t < KVC_WAVE; t++) {
+            const float v0 = lo(raw[t]), v1 = hi(raw[t]);
+            mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
+            mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
+        }
+        g0 = kvc_group_params(mn0, mx0, a.eb);
+        g1 = kvc_group_params(mn1, mx1, a.eb);
+        const int8_t m0 = (int8_t)(int)g0.min_i, m1 = (int8_t)(int)g1.min_i;     // quantize with the minimum as it is stored
+        g0.min_i = (float)m0;
+        g1.min_i = (float)m1;
+        g0.min_h = __float2half_rn(g0.min_i);
+        g1.min_h = __float2half_rn(g1.min_i);
+        if (act) {
+            a.scale_f16[g] = g0.scale_h;
+            a.scale_f16[g + 1] = g1.scale_h;
+            a.min_i8[g] = m0;
+            a.min_i8[g + 1] = m1;
+        }
+    } else {                                             // one pair per 64-token block (kernels.cu:771-772)
+        g0 = g1 = kvc_stored_params(a, row);
+    }
+    if (act) {
+#pragma unroll
+        for (int t = 0; t < KVC_WAVE; t++) {
+            const uint32_t s2 = (uint32_t)kvc_quant_one(lo(raw[t]), g0) | ((uint32_t)kvc_quant_one(hi(raw[t]), g1) << 8);
+            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)s2;
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int nd = D >> 2;
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
+}
+
 // V tile: 128 tokens x 64 flat channels.  While the tile is quantized, lane l owns channels 2 (l & 31), + 1 of
 // tokens 64 (l >> 5) .. + 63 (one load instruction = two tokens' runs of 64 halves); four tokens' symbols of a
 // channel are gathered in a register and written to LDS as one word of the [channel][token] tile, and lane c
@@ -566,7 +644,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
     __syncthreads();
     if (tile < a.e.tiles) {
         uint32_t v[32];
-        if (IS_K) kvc_front_k<true>(a, tile, lane, s_sym[wave], v);
+        if (IS_K) kvc_front_k_once(a, tile, lane, s_sym[wave], v);
         else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
         const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len[wave], &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
@@ -599,7 +677,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
     for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
     kvc_wave_lds_sync();
-    kvc_pack_vector(a.e, tile, lane, v, s_table[wave], image, p.head, s_short[wave] != 0u);
+    kvc_pack_vector(a.e, kvc_stream_start(a.e, tile, lane), v, s_table[wave], image, p.head, s_short[wave] != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a.e, p, lane, image);
 }

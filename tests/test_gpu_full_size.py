@@ -2,8 +2,9 @@
 decode(encode(quantize(x))) returns the quantizer's symbols exactly, the fused store produces the same stream
 as quantize-then-encode, decode + dequantize equals the dequantized symbols bit for bit and stays inside the
 error bound, and decode attention on the compressed cache matches fp32 PyTorch attention over the dequantized
-cache within 1e-3 of max|reference|.  Inputs are the synthetic distributions of the benchmark, generated on
-the device."""
+cache within 1e-3 of max|reference|.  Inputs are the synthetic distributions of the benchmark (the seeded host
+generators of tests/_synth.py, as bench.py uses them); the long-context configuration runs at each of its three K
+error bounds."""
 import math
 
 import pytest
@@ -17,6 +18,8 @@ CONFIGS = {
     "cfg2": (1, 32, 32, 128, 4096, 0.1, 0.2, "gauss"),
     "cfg3": (16, 8, 32, 128, 8192, 0.1, 0.2, "gauss"),
     "cfg5": (4, 32, 32, 96, 32768, 0.1, 0.3, "laplace"),
+    "cfg5_eb_k_0.05": (4, 32, 32, 96, 32768, 0.05, 0.3, "laplace"),
+    "cfg5_eb_k_0.2": (4, 32, 32, 96, 32768, 0.2, 0.3, "laplace"),
 }
 
 
@@ -27,7 +30,7 @@ def _make(name):
     return bench.make_kv(cfg, torch.device(DEV))
 
 
-@pytest.mark.parametrize("name", ["cfg2", "cfg3", "cfg5"])
+@pytest.mark.parametrize("name", list(CONFIGS))
 def test_full_size_round_trip_and_attention(name):
     from kvcomp_amd.attention import CompressedAttention
     from kvcomp_amd.compute import QuantMode, dequant, quant
@@ -71,7 +74,10 @@ def test_full_size_round_trip_and_attention(name):
         out = CompressedAttention(kctx, vctx).attend(q)
         out_r = None
         _lib.set_option("fused_rounded", 1)
-        out_r = CompressedAttention(kctx, vctx).attend(q)
+        out_r = CompressedAttention(kctx, vctx).attend(q)              # matrix-core kernels
+        was_m = _lib.set_option("fused_mfma", 0)
+        out_rf = CompressedAttention(kctx, vctx).attend(q)             # the same arithmetic on the fp32-FMA kernels
+        _lib.set_option("fused_mfma", was_m)
     finally:
         _lib.set_option("fused_rounded", was)
     rep = Hq // H
@@ -104,3 +110,6 @@ def test_full_size_round_trip_and_attention(name):
     # (3) In rounded mode the kernels round each dequantized value to fp16 first, like that dequantizer: then they
     #     meet the fp16-cache reference itself within 1e-3 of max|reference|.
     assert float((out_r.double() - ref_fp16).abs().max()) <= 1e-3 * scale
+    assert float((out_rf.double() - ref_fp16).abs().max()) <= 1e-3 * scale
+    # ... element by element too: within 1e-3 of the value, or of the output's typical size for the smallest ones
+    assert torch.allclose(out_r.double(), ref_fp16, rtol=1e-3, atol=1e-3 * float(ref_fp16.pow(2).mean().sqrt()))
