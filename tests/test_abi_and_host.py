@@ -41,6 +41,19 @@ def test_missing_library_fails_loudly(monkeypatch):
         _lib.lib()
 
 
+def test_the_reference_module_name_resolves_to_this_library():
+    """`import kvcomp_cuda` (kvcomp_cuda_extension/kvcomp_cuda.pyi): four constants and nine functions."""
+    import kvcomp_cuda
+    from kvcomp_amd import kvcomp_cuda as impl
+    assert (kvcomp_cuda.K_VEC_LEN, kvcomp_cuda.K_VEC_PER_BLK, kvcomp_cuda.V_VEC_LEN, kvcomp_cuda.V_VEC_PER_BLK) == (128, 64, 128, 64)
+    for name in ("build_codebook", "calculate_buffer_size", "k_entropy_encode_cuda_export", "v_entropy_encode_cuda_export",
+                 "k_entropy_decode_cuda_export", "v_entropy_decode_cuda_export", "k_decode_and_mat_vec_mul_cuda_export",
+                 "v_decode_and_mat_vec_mul_cuda_export", "k_mat_vec_mul_cuda_export"):
+        assert getattr(kvcomp_cuda, name) is getattr(impl, name), name
+    x = torch.zeros(2, 128, 2, 2, 64, dtype=torch.uint8)
+    assert kvcomp_cuda.calculate_buffer_size(x, False, 2, 64) == impl.calculate_buffer_size(x, False, 2, 64)
+
+
 def test_calculate_buffer_size_matches_reference_formula():
     """src/kernels.cu:893-917."""
     import kvcomp_amd.kvcomp_cuda as m
