@@ -370,6 +370,8 @@ def main():
     ap.add_argument("--eb-k", type=float, default=None, help="override the K error bound of the workload (cfg5 sweeps 0.05 / 0.1 / 0.2)")
     ap.add_argument("--no-unrounded", action="store_true",
                     help="skip the extra pass in unrounded mode (keeps a kernel trace of this run to one variant per kernel)")
+    ap.add_argument("--settle-seconds", type=float, default=0.5,
+                    help="untimed run of the operator before warm-up, so the timed steps see the sustained clock")
     ap.add_argument("--no-sweep", action="store_true", help="cfg5: skip the sweep over K's error bound")
     ap.add_argument("--sync-store", action="store_true",
                     help="cfg4: wait for the device after every encode (the reference's behaviour) instead of queuing it")
@@ -481,6 +483,7 @@ def main():
     n_copies = len(attns)
     # Before anything is timed: the operator against fp32 attention over the fp16 cache the reference's dequantizer
     # gives (models/cache/kvcomp_encode.py:146), on one (batch, head) slice of this very cache, within 1e-3.
+    _lib.set_option("fused_rounded", 1)          # the headline is this mode, whatever the environment preset
     check = attns[0].attend(q)
     kd = kctx.get_only_compressed()[0][:, 0, 0].float()
     vd = vctx.get_only_compressed()[0][:, 0, 0].float()
@@ -492,6 +495,14 @@ def main():
     del kd, vd
     log("[bench] checked against fp32 attention over the dequantized cache (batch 0, KV head 0): max error %.1e of max|out|" % err)
 
+    # The card idles at a low clock while the host prepares inputs and takes some hundred milliseconds of work to
+    # reach its sustained one (the same pass, timed later in this run, was 8 - 10 % faster than when timed first):
+    # the operator runs untimed for a moment, then come the --warmup steps and the timed ones.
+    t_end = time.perf_counter() + args.settle_seconds
+    while time.perf_counter() < t_end:
+        for a in attns:
+            a.attend(q)
+        torch.cuda.synchronize()
     res = time_steps(attns, args.steps, args.warmup)
     ms_per_step, k_ms, v_ms = res["ms_per_step"], res["k_ms"], res["v_ms"]
     log("[bench] step %.3f ms (events: median %.3f, p10 %.3f, p90 %.3f) over %d copies of the cache; fused K kernel %.3f ms "
@@ -584,6 +595,7 @@ def main():
                                         "fp16_equivalent_GBs": round(4 * numel / (ms_per_step * 1e-3) / 1e9, 1),
                                         "pct_hbm_peak": round(100 * value / HBM_PEAK_GBS, 2),
                                         "event_ms_per_step": res["event_ms"], "cache_copies_cycled": n_copies,
+                                        "untimed_settle_seconds": args.settle_seconds,
                                         "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)},
                                         "arithmetic": "every (sym + min) * scale rounded to fp16 as the reference's dequantizer rounds it "
                                                       "(models/cache/kvcomp_encode.py:146), fp32 accumulation: within 1e-3 of fp32 attention over "

@@ -88,9 +88,9 @@ class CompressedAttention:
         # decode tables follow the contexts' codebooks (built once, rebuilt if a codebook is replaced)
         # (a context has no codebook until its first block is compressed)
         if self.k.decode_codebook is not None and self._k_lut_src is not self.k.decode_codebook:
-            self._k_lut, self._k_lut_src = build_lut(self.k.decode_codebook), self.k.decode_codebook
+            self._k_lut, self._k_lut_src = build_lut(self.k.decode_codebook, self.k.tree_format), self.k.decode_codebook
         if self.v.decode_codebook is not None and self._v_lut_src is not self.v.decode_codebook:
-            self._v_lut, self._v_lut_src = build_lut(self.v.decode_codebook), self.v.decode_codebook
+            self._v_lut, self._v_lut_src = build_lut(self.v.decode_codebook, self.v.tree_format), self.v.decode_codebook
         return self._k_lut, self._v_lut
 
     @staticmethod

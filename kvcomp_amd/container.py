@@ -62,7 +62,7 @@ def dumps(ctx: KVCompCtx) -> bytes:
         "quant_scale_rel": float(ctx.quant_scale_rel), "quant_dims": [int(d) for d in ctx.quant_dims],
         "block_size": ctx.block_size, "recent_size": ctx.recent_size,
         "ctx_len": ctx.ctx_len, "compressed_ctx_len": ctx.compressed_ctx_len,
-        "max_code_bits": ctx.max_code_bits, "max_tile_bytes": ctx.max_tile_bytes, "max_stream_bytes": ctx.max_stream_bytes,
+        "tree_format": ctx.tree_format, "max_code_bits": ctx.max_code_bits, "max_tile_bytes": ctx.max_tile_bytes, "max_stream_bytes": ctx.max_stream_bytes,
         "config": str(cfg) if cfg is not None else None,
         "sections": [],
     }
@@ -171,6 +171,9 @@ def check_consistency(header: dict):
             fail("%s holds %d values, the stream has %d quantization groups" % (name, numel(name), groups))
     if comp and (not numel("encoded_data") or not numel("decode_codebook") or not numel("encode_codebook")):
         fail("a compressed part without payload or codebook")
+    fmt = header.get("tree_format", 3)                     # absent in files written before the field existed: int8 nodes
+    if fmt not in (3, 5) or numel("decode_codebook") % fmt:
+        fail("decode tree of %d bytes in node format %r" % (numel("decode_codebook"), fmt))
     tail_shape = list(secs["tail"]["shape"]) if secs["tail"]["nbytes"] else [0, B, H, D]
     if tail_shape != [total - comp, B, H, D]:
         fail("the tail has shape %s, expected %s" % (tail_shape, [total - comp, B, H, D]))
@@ -202,6 +205,7 @@ def loads(data: bytes, device: Optional[torch.device] = None) -> KVCompCtx:
             store.append(tensors[name])
     ctx.encode_codebook = tensors["encode_codebook"]
     ctx.decode_codebook = tensors["decode_codebook"]
+    ctx.tree_format = int(header.get("tree_format", 3))
     if tensors["tail"] is not None:
         ctx._tail_append(tensors["tail"])
     ctx.ctx_len = header["ctx_len"]

@@ -53,6 +53,16 @@ constexpr int kvc_fused_occupancy(int rep, int kind)
 #ifndef KVC_FUSED_OCC
 #define KVC_FUSED_OCC(REP, KIND) kvc_fused_occupancy(REP, KIND)
 #endif
+#ifndef KVC_MFMA_OCC_K1
+#define KVC_MFMA_OCC_K1 7
+#endif
+#ifndef KVC_MFMA_OCC_V1
+#define KVC_MFMA_OCC_V1 6
+#endif
+constexpr int kvc_fused_mfma_occupancy(int rep, int kind)
+{
+    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : KVC_MFMA_OCC_V1) : kvc_fused_occupancy(rep, kind);
+}
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
 

@@ -63,7 +63,10 @@ __device__ __forceinline__ kvc_f4 kvc_mfma4(uint32_t a01, uint32_t a23, kvc_w2 b
 template <bool BCAST>
 __device__ __forceinline__ kvc_w2 kvc_read_columns(uint32_t addr, bool holder)
 {
-    kvc_w2 b = {0u, 0u};
+    kvc_w2 b;
+    // whatever the registers hold: with the broadcast the matrix core reads the operand from the first sixteen lanes
+    // and from no other, so the rest need no defined value (and no instruction to give them one)
+    asm volatile("" : "=v"(b.x), "=v"(b.y));
     if (!BCAST || holder) b = *(const kvc_lds_w2 *)(uintptr_t)addr;
     return b;
 }
@@ -216,6 +219,7 @@ __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32
                                              uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM], bool holder)
 {
     static_assert((2 * G) % 4 == 0, "whole groups of four per refill");
+    asm volatile("" : "+v"(msptr));      // kept in a vector register: one add per round instead of a move per read
     for (int i = 0; i < n; i += 2 * G) {
         const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
         const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
@@ -252,6 +256,7 @@ template <int PG, bool SKEW, int NM, bool ROUNDED, bool BCAST>
 __device__ __forceinline__ void kvc_mfma_pair_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t maskp, int n,
                                                   uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM], bool holder)
 {
+    asm volatile("" : "+v"(msptr));      // kept in a vector register: one add per round instead of a move per read
     for (int i = 0; i < n; i += 4 * PG) {
         const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
         const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
@@ -349,7 +354,7 @@ __device__ __forceinline__ float kvc_quad_next(float v)
 }
 
 template <int REP, int KIND, bool ROUNDED>
-__global__ void __launch_bounds__(KVC_WG, KVC_FUSED_OCC(REP, KIND)) kvc_fused_mfma_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) kvc_fused_mfma_kernel(KvcFusedArgs a)
 {
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;

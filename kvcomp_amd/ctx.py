@@ -18,6 +18,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from . import kvcomp_cuda
+from ._lib import KvcompError
 from .compute import (QUANT_MODE_MAP, QuantMode, blocks_to_compress, cut_tensor_ctx_len_0, dequant, dims_to_mask,  # noqa: F401
                       mask_keepdim_shape, quant, safe_cat)
 
@@ -194,6 +195,9 @@ class KVCompCtx:
         self.max_stream_bytes = 0          # longest lane stream seen so far (sizes the fused decoders' LDS rows)
         self.encode_codebook: Optional[torch.Tensor] = None
         self.decode_codebook: Optional[torch.Tensor] = None
+        # node layout of decode_codebook: the reference's 3-byte nodes (include/huffman.h:18-22) while the code fits them
+        # (at most 128 nodes, symbols up to 127), else 5-byte nodes; every decoder of this context is told which
+        self.tree_format = kvcomp_cuda.TREE_I8
         # what encodes that nobody waited for have left on the device: words 0 - 7 are kvc_encode_async's result words,
         # word 8 counts the payload bytes in _encoded; _enc_pending bounds the bytes the host has not learnt of yet
         self._state: Optional[torch.Tensor] = None
@@ -346,18 +350,16 @@ class KVCompCtx:
         bi_buf, ti_buf, idx_buf, payload_buf = self._scratch(sizes)
         codebook = None
         if self.encode_codebook is None:     # first stored chunk defines the codebook (kvcomp_encode.py:99-103)
+            counts = kvcomp_cuda.symbol_counts([quant_ints])
             if self.codebook_smoothing:
-                codebook = self._smoothed_codebook(quant_ints)
-            else:
-                shift, enc, dec = kvcomp_cuda.build_codebook([quant_ints])
-                assert shift == 0, "shift must be 0"
-                codebook = (enc, dec)
+                counts[:self._smoothed_symbols()] += 1
+            codebook = self._host_codebook(counts)
         enc_table = self.encode_codebook if codebook is None else codebook[0].to(self.device)
         fn = kvcomp_cuda.k_entropy_encode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_encode_cuda_export
         encoded_, block_infos_, vec_infos_ = fn(quant_ints, enc_table, bi_buf, ti_buf, idx_buf, payload_buf,
                                                 self._encoded.used, self.head_num, self.head_dim)
         if codebook is not None:
-            self._set_codebook(*codebook)
+            self._set_codebook(*codebook[:2], tree_format=codebook[2])
         self.max_tile_bytes = max(self.max_tile_bytes, kvcomp_cuda.last_encode_max_tile_bytes)
         self.max_stream_bytes = max(self.max_stream_bytes, kvcomp_cuda.last_encode_max_stream_bytes)
         self._append_encoded(encoded_)
@@ -416,21 +418,27 @@ class KVCompCtx:
         counts = kvcomp_cuda.symbol_counts_chunks(quant_ints.reshape(-1), 1)
         if self.codebook_smoothing:
             counts[0, :self._smoothed_symbols()] += 1
-        enc, trees, meta = kvcomp_cuda.build_codebook_device(counts)
         T = quant_ints.shape[0] * quant_ints.shape[1]
         before = (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len)
-        self._encode_direct(T, tables=enc, table_bytes=enc.shape[1], symbols=quant_ints, meta=meta, min_ints=min_ints,
-                            quant_scale=quant_scale)
-        try:
-            self._sync_sizes()
-        except Exception:
-            (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len) = before
-            self._state[1] = 0                                 # the error has been reported; the context is as it was
-            raise
+        for fmt in (kvcomp_cuda.TREE_I8, kvcomp_cuda.TREE_I16):
+            enc, trees, meta = kvcomp_cuda.build_codebook_device(counts, fmt)
+            self._encode_direct(T, tables=enc, table_bytes=enc.shape[1], symbols=quant_ints, meta=meta, min_ints=min_ints,
+                                quant_scale=quant_scale)
+            try:
+                self._sync_sizes()
+                break
+            except Exception:
+                (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len) = before
+                self._state[1] = 0                             # the error has been reported; the context is as it was
+                self._enc_pending = 0
+                # status 4: the code does not fit the int8 tree (kvc_build_codebook_device) -- once more with the wide one
+                if fmt == kvcomp_cuda.TREE_I8 and int(meta[0, 3]) == 4:
+                    continue
+                raise
         self._encoded.trim()                                   # a byte per symbol was reserved; the stream is a fraction of it
         shift, enc_bytes, dec_bytes, status = (int(v) for v in meta[0].cpu())
         assert status == 0 and shift == 0, "shift must be 0"
-        self._set_codebook(enc[0, :enc_bytes].cpu(), trees[0, :dec_bytes].cpu())
+        self._set_codebook(enc[0, :enc_bytes].cpu(), trees[0, :dec_bytes].cpu(), tree_format=fmt)
 
     def _smoothed_symbols(self) -> int:
         return min(256, int(math.ceil(1.0 / self.quant_scale_rel)) + 3)      # symbols 0 .. ceil(1 / eb) + 2
@@ -441,13 +449,17 @@ class KVCompCtx:
     # occurs, so all of them get a code; the codebook then differs from the reference's for the same chunk.
     codebook_smoothing = False
 
-    def _smoothed_codebook(self, quant_ints: torch.Tensor):
-        n_sym = self._smoothed_symbols()
-        counts = kvcomp_cuda.symbol_counts([quant_ints])
-        counts[:n_sym] += 1
-        shift, enc, dec = kvcomp_cuda.build_codebook_from_counts(counts)
+    def _host_codebook(self, counts: torch.Tensor):
+        """(encode table, decode tree, tree format) from 256 symbol counts, by the host builder: the reference's int8
+        tree where the code fits it, the int16 tree where it does not (more than 64 symbols, or one above 127)."""
+        try:
+            shift, enc, dec = kvcomp_cuda.build_codebook_from_counts(counts, kvcomp_cuda.TREE_I8)
+            fmt = kvcomp_cuda.TREE_I8
+        except KvcompError:
+            shift, enc, dec = kvcomp_cuda.build_codebook_from_counts(counts, kvcomp_cuda.TREE_I16)
+            fmt = kvcomp_cuda.TREE_I16
         assert shift == 0, "shift must be 0"
-        return enc, dec
+        return enc, dec, fmt
 
     def _store_fused(self, to_compress: torch.Tensor, mask: int):
         """fp16 rows -> payload + metadata in one call (kvc_store_fused); same outputs as the two-step path."""
@@ -487,7 +499,7 @@ class KVCompCtx:
                               self.head_num, self.head_dim, dtype=torch.uint8, device=self.device)
         fn = kvcomp_cuda.k_entropy_decode_cuda_export if self.is_k else kvcomp_cuda.v_entropy_decode_cuda_export
         t_ms = fn(self.encoded_data, self.block_infos, self.thread_infos, self.decode_codebook, decoded,
-                  self.head_num, self.head_dim)
+                  self.head_num, self.head_dim, self.tree_format)
         return decoded, t_ms
 
     # decode and dequantize in one kernel (no uint8 tensor in between); False = the reference's two steps
@@ -501,7 +513,7 @@ class KVCompCtx:
                               device=self.device)
             t_ms = kvcomp_cuda.decode_dequant(self.is_k, self.encoded_data, self.block_infos, self.thread_infos,
                                               self.decode_codebook, self.quant_min_ints, self.quant_scales,
-                                              dims_to_mask(self.quant_dims), self.block_size, out)
+                                              dims_to_mask(self.quant_dims), self.block_size, out, self.tree_format)
             return out, t_ms
         decoded, t_ms = self.get_decode_quant_ints()
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -535,14 +547,16 @@ class KVCompCtx:
             C = torch.empty(self.batch_size, q_heads, self.compressed_ctx_len, dtype=torch.float16, device=self.device)
             t_ms = kvcomp_cuda.k_decode_and_mat_vec_mul_cuda_export(
                 self.decode_codebook, self.block_infos, self.thread_infos, self.encoded_data,
-                self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim)
+                self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim,
+                self.tree_format)
             return C, t_ms
         assert B.shape[2] == self.compressed_ctx_len, "ctx len mismatch"
         C = torch.empty(self.compressed_ctx_len // kvcomp_cuda.V_VEC_LEN, self.batch_size, q_heads, self.head_dim,
                         dtype=torch.float16, device=self.device)
         t_ms = kvcomp_cuda.v_decode_and_mat_vec_mul_cuda_export(
             self.decode_codebook, self.block_infos, self.thread_infos, self.encoded_data,
-            self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim)
+            self.quant_min_ints.reshape(-1), self.quant_scales.reshape(-1), B.contiguous(), C, self.head_num, self.head_dim,
+            self.tree_format)
         start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         start.record()
         C = C.sum(dim=0, keepdim=True, dtype=torch.float32).to(torch.float16)
@@ -561,15 +575,15 @@ class KVCompCtx:
             blocked_len = cache.shape[0] // self.block_size * self.block_size
             blocked = cache[:blocked_len].reshape(-1, self.block_size, self.batch_size, self.head_num, self.head_dim)
             sym.append(quant(blocked, self.quant_dims, self.quant_scale_rel)[0])
-        shift, enc, dec = kvcomp_cuda.build_codebook(sym)
-        assert shift == 0, "shift must be 0"
+        enc, dec, fmt = self._host_codebook(kvcomp_cuda.symbol_counts(sym))
         if self.device is None:
             self.device = device_
             KVCompCtx.buffer_ctx_len[self.device] = 0
-        self._set_codebook(enc, dec)
+        self._set_codebook(enc, dec, tree_format=fmt)
 
-    def _set_codebook(self, enc: torch.Tensor, dec: torch.Tensor):
+    def _set_codebook(self, enc: torch.Tensor, dec: torch.Tensor, tree_format: int = kvcomp_cuda.TREE_I8):
         """enc / dec: CPU byte tensors from kvcomp_cuda.build_codebook."""
+        self.tree_format = tree_format
         lengths = enc.view(torch.int32)[1::2]
         self.max_code_bits = int(lengths.max())      # sizes the fused decoders' table in LDS
         self.encode_codebook = enc.to(self.device)

@@ -16,6 +16,7 @@ class _Stub:
     batch_size, head_num, head_dim = 1, 2, 8
     quant_scale_rel, quant_dims, block_size, recent_size = 0.1, [1], 64, 64
     ctx_len, compressed_ctx_len, max_code_bits, max_tile_bytes, max_stream_bytes = 70, 64, 5, 100, 9
+    tree_format = 3
     encode_codebook = torch.arange(16, dtype=torch.uint8)
     decode_codebook = torch.arange(6, dtype=torch.uint8)
     block_infos = torch.zeros(16, dtype=torch.uint8)

@@ -355,6 +355,50 @@ def test_one_call_attention_grows_with_the_cache(fused_mode):
             assert (out - ref).abs().max() <= fused_mode.tol_vs_fp16_cache * ref.abs().max(), "step %d" % i
 
 
+@pytest.mark.parametrize("device_codebook", [True, False])
+def test_a_fine_error_bound_falls_back_to_the_wide_tree(device_codebook):
+    """More than 64 symbols do not fit the reference's int8 decode tree (include/huffman.h:18-22): the context then
+    keeps a 5-byte-node tree and tells every decoder, instead of failing the store and every store after it."""
+    from kvcomp_amd import container, kvcomp_cuda
+    from kvcomp_amd.attention import CompressedAttention
+    from kvcomp_amd.compute import dequant
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant")
+    T, B, H, D = 512, 1, 2, 128
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.004), KVCompCtx(False, B, H, D, 0.2)
+    kctx.device_codebook = device_codebook
+    sym = kctx.store(k)
+    vctx.store(v)
+    assert int(sym.max()) > 127 and kctx.tree_format == kvcomp_cuda.TREE_I16 and vctx.tree_format == kvcomp_cuda.TREE_I8
+    assert kctx.decode_codebook.numel() % 5 == 0
+    # the host builder's wide tree for the same counts, byte for byte
+    _, enc, dec = kvcomp_cuda.build_codebook([sym], kvcomp_cuda.TREE_I16)
+    assert torch.equal(kctx.encode_codebook.cpu(), enc) and torch.equal(kctx.decode_codebook.cpu(), dec)
+    dec_sym, _ = kctx.get_decode_quant_ints()
+    assert torch.equal(dec_sym, sym)
+    full, _ = kctx.get_only_compressed()
+    ref = dequant(sym, kctx.quant_min_ints, kctx.quant_scales, kctx.quant_dims).flatten(0, 1)
+    assert torch.equal(full.view(torch.int16), ref.view(torch.int16))
+    again = kctx.store(k)                                    # a second store with the codebook in place
+    assert torch.equal(again, sym) and kctx.compressed_ctx_len == 2 * T
+    vctx.store(v)
+    q = S.synth_q(B, H, D).to(DEV)
+    out = CompressedAttention(kctx, vctx).attend(q)
+    kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+    s = torch.einsum("tbhd,bhd->bht", kd, q.float()) / D ** 0.5
+    want = torch.einsum("tbhd,bht->bhd", vd, torch.softmax(s, dim=-1))
+    assert (out - want).abs().max() <= 1e-3 * want.abs().max()
+    assert torch.equal(kctx.mat_vec_mul(q)[0].float(), kctx.mat_vec_mul(q)[0].float())
+    scores = kctx.mat_vec_mul(q)[0].float()
+    dense = torch.einsum("tbhd,bhd->bht", kd, q.float())
+    assert (scores - dense).abs().max() <= 2e-3 * dense.abs().max()       # fp16 scores out
+    # the container carries the node format
+    back = container.loads(container.dumps(kctx), DEV)
+    assert back.tree_format == kvcomp_cuda.TREE_I16
+    assert torch.equal(back.get_only_compressed()[0], kctx.get_only_compressed()[0])
+
+
 @pytest.mark.parametrize("is_k,mode,B,H,D", [(True, "ChannelQuant", 2, 3, 96), (True, "BlockQuant", 1, 4, 128),
                                               (False, "TokenQuant", 2, 3, 96), (False, "VectorQuant", 2, 4, 128)])
 def test_one_kernel_get_equals_decode_then_dequant(is_k, mode, B, H, D):
