@@ -501,7 +501,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                     if (rr == r) bs = bias[rr];
 #pragma unroll
                 for (int i = 0; i < 4; i++)
-                    res[i] = fmaf(kvc_quad_next(acc[s][i]), 1.f / KVC_LO_SCALE, acc[s][i]) * unscale + bs;
+                    res[i] = fmaf(kvc_quad_next(acc[s][i]), 1.f / KVC_LO_SCALE, acc[s][i]);
+                if (!ROUNDED) {                        // rounded mode folds nothing into a constant and never rescales
+#pragma unroll
+                    for (int i = 0; i < 4; i++) res[i] = res[i] * unscale + bs;
+                }
                 if ((j & 1) == 0 && r < REP) {
                     const int64_t o = out_base + r * out_step + rows4;
                     if (a.out_f32) {
