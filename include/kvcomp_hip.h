@@ -79,6 +79,11 @@ int kvc_abi_version(void);
  *   "fused_builtin_dpp":     0 (default): the fp32-FMA kernels pick their operand out of a quad of lanes with a permute
  *                           written as inline assembly on the multiply-add itself; 1: through the compiler's lane-
  *                           permute intrinsic (same result bit for bit; a cross-check against toolchain changes).
+ *   "fused_schedule":       -1 (default) decided per call: a matrix-core launch over a stream with one codebook and at
+ *                           least 32768 tiles walks the row-major tile sequence with runs of 4 tiles per wave for the
+ *                           first 70 % of the tiles, 2 for the next 20 %, single tiles last; 0: never (every wave
+ *                           takes "fused_tiles_per_wave" tiles of one tile row); r * 10000 + p * 100 + q: runs of r
+ *                           for the first p %, r / 2 for the next q %, r / 4 and 1 for halves of the rest.
  *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
  *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile

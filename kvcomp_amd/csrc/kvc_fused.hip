@@ -908,6 +908,8 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
 
 // Consecutive tiles of a row that one wave works through (fetching one ahead): as many as still leave
 // every SIMD of the chip several waves.
+constexpr int KVC_DEFAULT_SCHEDULE = 47020;      // runs of 4 for 70 % of the tiles, of 2 for 20 %, single tiles last
+
 static int kvc_plan_tiles_per_wave(int64_t tiles)
 {
     const int forced = kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE);
@@ -916,6 +918,48 @@ static int kvc_plan_tiles_per_wave(int64_t tiles)
     // decode of the first; 49 152 tiles: 3 % faster than one); at 16 384 tiles one is 3 % faster, and longer runs
     // only leave fewer workgroups to balance over the chip (8 per wave: 15 % slower)
     return tiles >= 32768 ? 2 : 1;
+}
+
+// Schedule of a matrix-core launch over `tiles` tiles (see KvcFusedArgs::sched_*): long runs of tiles per wave
+// first, so that most tiles share a wave's set-up and their fetches overlap the previous tile's decode, shorter ones
+// after, single tiles last, so that the last workgroups to start are short.  Returns the number of workgroups, 0 for
+// the plain 2-D grid.
+static unsigned kvc_plan_schedule(KvcFusedArgs &a, int64_t tiles)
+{
+    a.sched_nseg = 0;
+    int want = kvc_option(KVC_OPT_FUSED_SCHEDULE);
+    if (want == 0 || a.s.rows_per_codebook != 0 || tiles > (int64_t)1 << 30) return 0;
+    if (want < 0) {
+        if (tiles < 32768) return 0;      // few tiles: one or two per wave in the plain grid
+        want = KVC_DEFAULT_SCHEDULE;
+    }
+    const int run0 = want / 10000, pct0 = (want / 100) % 100, pct1 = want % 100;
+    if (run0 < 1 || run0 > 64 || pct0 + pct1 > 100) return 0;
+    const int per_wg[KVC_SCHED_SEGMENTS] = {run0, run0 / 2 > 1 ? run0 / 2 : 1, run0 / 4 > 1 ? run0 / 4 : 1, 1};
+    const int64_t rest = tiles - tiles * (pct0 + pct1) / 100;
+    int64_t want_tiles[KVC_SCHED_SEGMENTS] = {tiles * pct0 / 100, tiles * pct1 / 100, rest / 2, 0};
+    int64_t tile = 0, wg = 0;
+    int k = 0;
+    for (int i = 0; i < KVC_SCHED_SEGMENTS && tile < tiles; i++) {
+        const int64_t chunk = (int64_t)per_wg[i] * KVC_WAVES_PER_WG;
+        // whole workgroups; the last segment takes whatever is left
+        int64_t n = i == KVC_SCHED_SEGMENTS - 1 ? tiles - tile : want_tiles[i] / chunk * chunk;
+        if (n > tiles - tile) n = tiles - tile;
+        if (n <= 0) continue;
+        a.sched_run[k] = per_wg[i];
+        a.sched_wg[k] = (int)wg;
+        a.sched_tile[k] = (int)tile;
+        tile += n;
+        wg += (n + chunk - 1) / chunk;
+        k++;
+    }
+    a.sched_nseg = k;
+    for (int i = k; i <= KVC_SCHED_SEGMENTS; i++) {
+        a.sched_wg[i] = (int)wg;
+        a.sched_tile[i] = (int)tiles;
+        if (i < KVC_SCHED_SEGMENTS) a.sched_run[i] = 1;
+    }
+    return (unsigned)wg;
 }
 
 // what the one-call attention adds to a plain fused launch
@@ -1001,8 +1045,16 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     if (!d_luts) {
         if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
     }
-    const dim3 grid = kvc_grid(a.s, rows);
+    dim3 grid = kvc_grid(a.s, rows);
+    a.sched_nseg = 0;
+    if (mfma) {
+        if (const unsigned wgs = kvc_plan_schedule(a, rows * a.s.cols)) grid = dim3(wgs, 1);
+    }
     static const bool trace_plan = getenv("KVCOMP_TRACE_PLAN") != nullptr;
+    if (trace_plan && a.sched_nseg)
+        fprintf(stderr, "[kvcomp] schedule: %d segments, runs %d %d %d %d from workgroups %d %d %d %d (tiles %d %d %d %d), %d tiles\n",
+                a.sched_nseg, a.sched_run[0], a.sched_run[1], a.sched_run[2], a.sched_run[3], a.sched_wg[0], a.sched_wg[1],
+                a.sched_wg[2], a.sched_wg[3], a.sched_tile[0], a.sched_tile[1], a.sched_tile[2], a.sched_tile[3], a.sched_tile[4]);
     if (trace_plan)
         fprintf(stderr, "[kvcomp] fused kind %d rep %d: grid %u x %u, lds %zu B (table %d w, payload %d w of %d logical, "
                 "skew %d, rows %d), pair bits %d, tiles per wave %d, rounded %d\n", kind, (int)rep, grid.x, grid.y, lds,
@@ -1042,6 +1094,7 @@ int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_t
     void *slot = nullptr;
     if (int rc = kvc_workspace_slot(&slot)) return rc;
     KvcFusedArgs a;
+    a.sched_nseg = 0;
     int64_t rows;
     const int64_t stride = batch * heads * head_dim;
     if (int rc = kvc_fill_stream_args(a.s, d_encoded, encoded_bytes, d_block_infos, block_infos_bytes, d_thread_infos,

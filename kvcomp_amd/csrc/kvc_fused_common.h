@@ -6,6 +6,8 @@
 #include <mutex>
 #include <type_traits>
 
+constexpr int KVC_SCHED_SEGMENTS = 4;
+
 struct KvcFusedArgs {
     KvcStreamArgs s;
     const int8_t *min_i8;
@@ -39,6 +41,13 @@ struct KvcFusedArgs {
     int rounded;
     int expand;          // 0: matvec kernels; 1: symbols out (uint8); 2: dequantized values out (fp16)
     int out_words;       // LDS words per wave for the 32-element output slab
+    // Matrix-core kernels, one codebook per stream: 1-D grid over the row-major tile sequence in sched_nseg segments
+    // (0: the 2-D grid of kvc_grid).  Segment k = workgroups sched_wg[k] .. sched_wg[k + 1] - 1, whose waves take
+    // sched_run[k] consecutive tiles each, starting at tile sched_tile[k]; sched_tile[sched_nseg] = number of tiles.
+    int sched_nseg;
+    int sched_run[KVC_SCHED_SEGMENTS];
+    int sched_wg[KVC_SCHED_SEGMENTS + 1];
+    int sched_tile[KVC_SCHED_SEGMENTS + 1];
 };
 
 // Workgroups per CU (= waves per SIMD) each matvec kernel is compiled for.  With one query head per KV head the

@@ -82,6 +82,16 @@ __device__ __forceinline__ uint32_t kvc_dequant_pair(uint32_t x, uint32_t mn, ui
 // upper halves of two table entries side by side: {a >> 16, b >> 16 << 16}
 __device__ __forceinline__ uint32_t kvc_pack_hi16(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
+// The kernel's argument block read again from the kernarg segment (scalar loads that hit the scalar cache): what a
+// tile needs of it is then live only where it is used, not in scalar registers through the decode loops.
+template <class T>
+__device__ __forceinline__ const T &kvc_kernarg_again()
+{
+    auto p = __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return *(const T *)p;
+}
+
 // -- operand tables -----------------------------------------------------------------------------------
 // btab  [slot][group g][set][column j][element k]  fp16: weight part of element 4 g + k for column 4 set + j;
 //       column 2 r is the high part of query head r's weight, column 2 r + 1 its low part times 4096
@@ -354,8 +364,9 @@ __device__ __forceinline__ float kvc_quad_next(float v)
 }
 
 template <int REP, int KIND, bool ROUNDED>
-__global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) kvc_fused_mfma_kernel(KvcFusedArgs a)
+__global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) kvc_fused_mfma_kernel(KvcFusedArgs a_in)
 {
+    const KvcFusedArgs &a = a_in;
     constexpr bool IS_K = KIND == 0;
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     constexpr int NM = kvc_mfma_sets(REP);
@@ -371,8 +382,39 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     uint32_t *btab = smem + a.table_words + wave * per_wave;
     uint32_t *mstab = btab + SLOTS * T::BTAB_SLOT_WORDS;
     uint32_t *pack = btab + OPS_WORDS;
-    const int row = blockIdx.y;
-    const int64_t cb = a.s.rows_per_codebook ? row / a.s.rows_per_codebook : 0;
+    // Which tiles this wave takes.  Plain launch: grid (column groups, tile rows), every wave `tiles_per_wave`
+    // consecutive columns of its row.  Scheduled launch (sched_nseg > 0; one codebook for the whole stream): a 1-D grid
+    // over the row-major tile sequence in a few segments, the waves of segment k taking sched_run[k] consecutive tiles
+    // each; runs shorten towards the end of the launch, so that most tiles share a wave's set-up with several others
+    // while the last workgroups to start are short and the chip drains quickly.
+    int t_first, ntiles;
+    const int cols = a.s.cols;
+    if (a.sched_nseg) {
+        const int wg = blockIdx.x;
+        int k = 0;
+#pragma unroll
+        for (int i = 1; i < KVC_SCHED_SEGMENTS; i++)
+            if (i < a.sched_nseg && wg >= a.sched_wg[i]) k = i;
+        const int run = a.sched_run[k];
+        t_first = a.sched_tile[k] + ((wg - a.sched_wg[k]) * KVC_WAVES_PER_WG + wave) * run;
+        ntiles = a.sched_tile[k + 1] - t_first;
+        ntiles = ntiles < run ? ntiles : run;
+    } else {
+        const int TPW = a.s.tiles_per_wave;
+        const int c0 = (blockIdx.x * KVC_WAVES_PER_WG + wave) * TPW;
+        t_first = blockIdx.y * cols + c0;
+        ntiles = cols - c0;
+        ntiles = ntiles < TPW ? ntiles : TPW;
+    }
+    int row = t_first / cols, col = t_first - row * cols;
+    // block_info of the wave's j-th tile in lane j (asked for before the table is set up: the two waits overlap)
+    uint32_t bi_off = 0, bi_bn = 0;
+    if (lane < ntiles) {
+        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.s.block_infos + 8 * ((int64_t)t_first + lane));
+        bi_off = bi[0];
+        bi_bn = bi[1];
+    }
+    const int64_t cb = a.s.rows_per_codebook ? (a.sched_nseg ? 0 : (int)blockIdx.y) / a.s.rows_per_codebook : 0;
     const uint32_t *__restrict__ lut_g = a.s.luts + cb * KVC_LUT_WORDS;
     const uint32_t lbits = lut_g[0], lmax = lut_g[1], nlong = lut_g[2];
     const bool fast_book = nlong == 0 && lmax >= 1u && lmax <= 7u && (1u << lbits) <= (uint32_t)a.table_words;
@@ -386,8 +428,17 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     const uint32_t pbits = 2u * lmax;
     // two symbols per look-up: twice the longest code fits the index, and no symbol's fp16 pattern needs the five
     // bits the lengths of a two-symbol entry go to (header word 6: OR of all the patterns)
-    const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
+#ifdef KVC_EXP_KIND
+    constexpr bool EXPF = KIND == KVC_EXP_KIND && REP == 1 && ROUNDED;
+#else
+    constexpr bool EXPF = false;
+#define KVC_EXP_PAIRS 0
+#define KVC_EXP_PER 12
+#define KVC_EXP_SKEW 0
+#endif
+    const bool pairs_rt = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
                        (1u << pbits) <= (uint32_t)a.table_words && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
+    const bool pairs = EXPF ? (bool)KVC_EXP_PAIRS : pairs_rt;
     if (pairs) {
         // the one-symbol table goes to the (not yet used) per-wave areas; the two-symbol table is derived from it
         uint32_t *tmp = smem + a.table_words;
@@ -410,42 +461,34 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     const uint32_t mask4 = ((1u << lbits) - 1u) << 2, maskp = ((1u << pbits) - 1u) << 2;
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
     // symbols per refill in the main part (a multiple of four); what is left goes eight per refill
-    const int per = pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
+    const int per = EXPF ? KVC_EXP_PER : pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
     int n_main = (n / per) * per;
     while ((n - n_main) % 8 != 0) n_main -= per;
     const uint32_t fe = kvc_lds_addr(smem);                            // 0: the table opens the workgroup's LDS
 
-    // this wave's tiles: T consecutive columns of one tile row
-    const int TPW = a.s.tiles_per_wave;
-    const int col0 = (blockIdx.x * KVC_WAVES_PER_WG + wave) * TPW;
-    int ntiles = a.s.cols - col0;
-    ntiles = ntiles < TPW ? ntiles : TPW;
     if (ntiles <= 0) return;
-    // block_info of tile col0 + j in lane j
-    uint32_t bi_off = 0, bi_bn = 0;
-    if (lane < ntiles) {
-        const uint32_t *bi = reinterpret_cast<const uint32_t *>(a.s.block_infos + 8 * ((int64_t)row * a.s.cols + col0 + lane));
-        bi_off = bi[0];
-        bi_bn = bi[1];
-    }
     KvcRaw<REP, SLOTS, KvcGeom<KIND>::XW> raw;
-    kvc_fetch_tile<REP, KIND>(a, row, col0, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    kvc_fetch_tile<REP, KIND>(a, row, col, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
     float bias[REP], unscale;
     int sel = 0;
     uint32_t first, longest;
     KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
     if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;       // two bits before the lane's first code
-    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col0, lane, raw, btab, mstab, bias, unscale, sel);
+    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col, lane, raw, btab, mstab, bias, unscale, sel);
     kvc_wave_sync();
     for (int it = 0; it < ntiles; it++) {
-        const int col = col0 + it;
+        // the arguments are read again per tile rather than kept in scalar registers through the decode loops (the
+        // kernel needs more scalars than there are registers, and every spilled one costs a vector instruction)
+        const KvcFusedArgs &a = kvc_kernarg_again<KvcFusedArgs>();
         const bool more = it + 1 < ntiles;
+        int row_next = row, col_next = col + 1;        // row-major successor
+        if (col_next == cols) col_next = 0, row_next = row + 1;
         // the lane number is made opaque per tile, so that the addresses the fetch and the staging derive from it
         // are not kept in registers through the decode loops
         int lane_f = lane;
         asm volatile("" : "+v"(lane_f));
         if (more)   // loads for the next tile fly while this one is decoded
-            kvc_fetch_tile<REP, KIND>(a, row, col + 1, __builtin_amdgcn_readlane(bi_off, it + 1),
+            kvc_fetch_tile<REP, KIND>(a, row_next, col_next, __builtin_amdgcn_readlane(bi_off, it + 1),
                                       __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
         const uint32_t *my_btab = btab + sel * T::BTAB_SLOT_WORDS, *my_mstab = mstab + sel * T::MSTAB_SLOT_WORDS;
         // geometry of the results
@@ -486,7 +529,8 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                     if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                 }
             };
-            if (a.skew) run(std::true_type{});
+            if (EXPF) run(std::integral_constant<bool, (bool)KVC_EXP_SKEW>{});
+            else if (a.skew) run(std::true_type{});
             else run(std::false_type{});
             // register i of lane 4 b + j: row 4 b + i, column 4 set + j; the even columns take their low parts from
             // the lane to their right and carry the results of query head 2 set + j / 2
@@ -538,9 +582,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             asm volatile("" : "+v"(lane_s));
             st = kvc_stage_payload(a, lane_s, raw, pack, first, longest);
             if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;
-            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col + 1, lane_s, raw, btab, mstab, bias, unscale, sel);
+            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row_next, col_next, lane_s, raw, btab, mstab, bias, unscale, sel);
             kvc_wave_sync();
         }
+        row = row_next;
+        col = col_next;
     }
 }
 
