@@ -73,9 +73,9 @@ int kvc_abi_version(void);
  *                           result is the fp32 attention over that fp16 cache (within 1e-3).  0: the product is used
  *                           as it stands, in fp32 (closer to exact arithmetic over the unrounded dequantization, and
  *                           further from the reference's cache: a few 1e-3 on outlier-heavy data).
- *   "fused_mfma":           -1 (default): the multiply-accumulate of the fused matvecs runs on the matrix cores
- *                           (v_mfma_f32_4x4x4_16b_f16) where that is the faster kernel (rounded mode, codes of at most
- *                           7 bits); 0 never; 1 wherever the matrix-core kernels apply.
+ *   "fused_mfma":           -1 (default) or 1: the multiply-accumulate of the fused matvecs runs on the matrix cores
+ *                           (v_mfma_f32_4x4x4_16b_f16) wherever those kernels apply (codes of at most 7 bits, results
+ *                           that can be stored four at a time); 0: never (fp32 multiply-adds on the vector units).
  *   "fused_builtin_dpp":     0 (default): the fp32-FMA kernels pick their operand out of a quad of lanes with a permute
  *                           written as inline assembly on the multiply-add itself; 1: through the compiler's lane-
  *                           permute intrinsic (same result bit for bit; a cross-check against toolchain changes).

@@ -1032,7 +1032,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     // skewed packed payload, results that can be stored four at a time.
     const int64_t out_stride = (extra && extra->out_stride) ? extra->out_stride : tokens;
     const int want_mfma = kvc_option(KVC_OPT_FUSED_MFMA);
-    const bool mfma = (want_mfma < 0 ? rounded != 0 : want_mfma != 0) && max_code_bits >= 1 && max_code_bits <= 7 &&
+    const bool mfma = want_mfma != 0 && max_code_bits >= 1 && max_code_bits <= 7 &&
                       kvc_option(KVC_OPT_FUSED_ROWS) != 1 && ((uintptr_t)d_out & 15) == 0 &&
                       (is_k ? out_stride % 4 == 0 : head_dim % 4 == 0);
     const size_t lds = mfma ? kvc_plan_lds(a, slots, (int)rep, encoded_bytes, rows * a.s.cols, max_tile_bytes, max_stream_bytes,

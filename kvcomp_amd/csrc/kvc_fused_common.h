@@ -63,7 +63,7 @@ constexpr int kvc_fused_occupancy(int rep, int kind)
 #define KVC_FUSED_OCC(REP, KIND) kvc_fused_occupancy(REP, KIND)
 #endif
 #ifndef KVC_MFMA_OCC_K1
-#define KVC_MFMA_OCC_K1 7
+#define KVC_MFMA_OCC_K1 8
 #endif
 #ifndef KVC_MFMA_OCC_V1
 #define KVC_MFMA_OCC_V1 6

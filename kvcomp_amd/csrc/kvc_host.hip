@@ -53,7 +53,7 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"decode_pipelined", "KVCOMP_DECODE_PIPELINED", 1},          // plain decode / decode + dequantize on the fused kernels' machinery
     {"fused_rounded", "KVCOMP_FUSED_ROUNDED", 1},                // 1: round each dequantized value to fp16 before the matvec, as the reference's dequantizer does
     {"attention_tail_in_merge", "KVCOMP_ATTENTION_TAIL_IN_MERGE", 1},   // kvc_attention_decode: V's fp16 tail inside the merge kernel
-    {"fused_mfma", "KVCOMP_FUSED_MFMA", -1},                     // matrix-core kernels: -1 where they are faster (rounded mode), 0 never, 1 always
+    {"fused_mfma", "KVCOMP_FUSED_MFMA", -1},                     // matrix-core kernels: -1 / 1 wherever they apply, 0 never
     {"fused_builtin_dpp", "KVCOMP_FUSED_BUILTIN_DPP", 0},        // fp32-FMA kernels: the quad permute through the compiler's intrinsic, not inline assembly
     {"fused_schedule", "KVCOMP_FUSED_SCHEDULE", -1},             // matrix-core kernels: runs of tiles per wave that shorten towards the end of the launch; -1 choose per call, 0 never, r * 10000 + p * 100 + q: runs of r for the first p % of the tiles, r / 2 for the next q %
 };

@@ -48,8 +48,8 @@ class FusedMode:
 
 FUSED_MODES = [FusedMode("rounded", 1, -1),            # the default: fp16-rounded dequantization, matrix-core kernels
                FusedMode("rounded_fma", 1, 0),         # the same arithmetic on the fp32-FMA kernels
-               FusedMode("unrounded", 0, -1),          # dequantized values left in fp32, fp32-FMA kernels
-               FusedMode("unrounded_mfma", 0, 1)]      # the same on the matrix-core kernels
+               FusedMode("unrounded", 0, 0),           # dequantized values left in fp32, fp32-FMA kernels
+               FusedMode("unrounded_mfma", 0, -1)]     # the same on the matrix-core kernels
 
 
 @pytest.fixture(params=FUSED_MODES, ids=[m.name for m in FUSED_MODES])

@@ -234,7 +234,7 @@ def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D, 
     # the plan changes where the bits are read from, not the arithmetic: results are identical, except that per-lane
     # rows are only implemented by the fp32-FMA kernels, whose sums are rounded in a different order than the
     # matrix cores' (both carry the products exactly)
-    same_kernel = rows == 0 or fused_mode.mfma == 0 or (fused_mode.mfma < 0 and not fused_mode.rounded)
+    same_kernel = rows == 0 or fused_mode.mfma == 0
     if same_kernel:
         assert torch.equal(out, default_plan)
     else:
