@@ -404,6 +404,27 @@ __device__ __forceinline__ void kvc_write_image(const KvcEncodeArgs &a, const Kv
     }
 }
 
+// The same for an image that was packed from its first word on, while the payload starts p.head bytes into an
+// aligned word of the destination: every output word is put together from two image words.
+__device__ __forceinline__ void kvc_write_image_shifted(const KvcEncodeArgs &a, const KvcEmitPlace &p, int lane, const uint32_t *image)
+{
+    uint8_t *dst = a.encoded + p.off - p.head;                 // 4-byte aligned
+    const uint32_t lo = p.head, hi = p.head + p.bn;            // valid byte range of the output words
+    const uint32_t nwords = (hi + 3u) >> 2;
+    const uint32_t shift = 8u * (4u - p.head);                 // 32, 24, 16, 8
+    for (uint32_t f = lane; f < nwords; f += KVC_WAVE) {
+        const uint32_t cur = f < (uint32_t)KVC_IMAGE_WORDS ? image[f] : 0u, prev = f ? image[f - 1] : 0u;
+        const uint32_t b0 = 4u * f, word = (uint32_t)((((uint64_t)cur << 32) | prev) >> shift);
+        if (b0 >= lo && b0 + 4u <= hi) {
+            reinterpret_cast<uint32_t *>(dst)[f] = word;
+        } else {
+#pragma unroll
+            for (uint32_t k = 0; k < 4; k++)
+                if (b0 + k >= lo && b0 + k < hi) dst[b0 + k] = (uint8_t)(word >> (8u * k));
+        }
+    }
+}
+
 __global__ void __launch_bounds__(KVC_WG) kvc_encode_emit_kernel(KvcEncodeArgs a)
 {
     __shared__ uint2 s_table[KVC_WAVES_PER_WG][256];
@@ -458,10 +479,10 @@ __device__ __forceinline__ KvcGroupParams kvc_stored_params(const KvcStoreArgs &
 // K tile: 64 tokens x D channels of one (batch, head).  Lane l owns channels 2l and 2l + 1 while the tile is
 // quantized (each load instruction of the wave is one token's contiguous run of D halves), the symbols go
 // to LDS as [token][channel], and lane t then reads token t's vector.
-// Per-channel groups live entirely inside the tile: the count pass (PUBLISH) finds min / max itself, writes
-// the group parameters and quantizes with exactly what it wrote (the minimum as int8), the emit pass reads
-// them back, so the two passes always agree.
-template <bool PUBLISH>
+// Per-channel groups live entirely inside the tile: the count pass (kvc_front_k_once) finds min / max itself, writes
+// the group parameters and quantizes with exactly what it wrote (the minimum as int8), the emit pass (kvc_front_k)
+// reads them back, so the two passes always agree.  Both quantize with packed fp16 arithmetic
+// (kvc_quant_pair_biased: two channels per instruction).
 __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t (&v)[32])
 {
     const int64_t stride = a.e.stride;
@@ -469,47 +490,20 @@ __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile,
     const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
     const bool act = 2 * lane < D;
     const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (act ? 2 * lane : 0);
-    auto lo = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); };
-    auto hi = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); };
     KvcGroupParams g0, g1;
     if (a.mask == KVC_MASK_CHANNEL) {
         const int64_t g = row * stride + col * D + (act ? 2 * lane : 0);
-        if (PUBLISH) {
-            // two walks over the tile's rows (the second one finds them in the cache) keep the register count low
-            float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
-#pragma unroll 8
-            for (int t = 0; t < KVC_WAVE; t++) {
-                const uint32_t w = *reinterpret_cast<const uint32_t *>(p + t * stride);
-                const float v0 = lo(w), v1 = hi(w);
-                mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
-                mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
-            }
-            g0 = kvc_group_params(mn0, mx0, a.eb);
-            g1 = kvc_group_params(mn1, mx1, a.eb);
-            const int8_t m0 = (int8_t)(int)g0.min_i, m1 = (int8_t)(int)g1.min_i;
-            g0.min_i = (float)m0;
-            g1.min_i = (float)m1;
-            g0.min_h = __float2half_rn(g0.min_i);
-            g1.min_h = __float2half_rn(g1.min_i);
-            if (act) {
-                a.scale_f16[g] = g0.scale_h;
-                a.scale_f16[g + 1] = g1.scale_h;
-                a.min_i8[g] = m0;
-                a.min_i8[g + 1] = m1;
-            }
-        } else {
-            g0 = kvc_stored_params(a, g);
-            g1 = kvc_stored_params(a, g + 1);
-        }
+        g0 = kvc_stored_params(a, g);
+        g1 = kvc_stored_params(a, g + 1);
     } else {                                             // one pair per 64-token block (kernels.cu:771-772)
         g0 = g1 = kvc_stored_params(a, row);
     }
+    const KvcPackedParams pp = kvc_packed_params(g0, g1);
     if (act) {
 #pragma unroll 8
         for (int t = 0; t < KVC_WAVE; t++) {
-            const uint32_t w = *reinterpret_cast<const uint32_t *>(p + t * stride);
-            const uint32_t s2 = (uint32_t)kvc_quant_one(lo(w), g0) | ((uint32_t)kvc_quant_one(hi(w), g1) << 8);
-            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)s2;
+            const uint32_t u = kvc_quant_pair_biased(*reinterpret_cast<const uint32_t *>(p + t * stride), pp);
+            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -521,7 +515,8 @@ __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile,
 }
 
 // The count pass's variant: the lane keeps its two channels of all 64 tokens in registers (64 loads in flight, one walk
-// over the tile instead of two), finds the groups' minima and maxima there, publishes the group parameters and quantizes.
+// over the tile), finds the groups' minima and maxima there (packed fp16 min / max), publishes the group parameters
+// and quantizes.
 __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t (&v)[32])
 {
     const int64_t stride = a.e.stride;
@@ -529,23 +524,22 @@ __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t 
     const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
     const bool act = 2 * lane < D;
     const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (act ? 2 * lane : 0);
-    auto lo = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w & 0xffffu))); };
-    auto hi = [](uint32_t w) { return __half2float(__ushort_as_half((unsigned short)(w >> 16))); };
     uint32_t raw[KVC_WAVE];
 #pragma unroll
     for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + t * stride);
     KvcGroupParams g0, g1;
     if (a.mask == KVC_MASK_CHANNEL) {
         const int64_t g = row * stride + col * D + (act ? 2 * lane : 0);
-        float mn0 = INFINITY, mx0 = -INFINITY, mn1 = INFINITY, mx1 = -INFINITY;
+        kvc_half2 mn = __builtin_bit_cast(kvc_half2, raw[0]), mx = mn;
 #pragma unroll
-        for (int t = 0; t < KVC_WAVE; t++) {
-            const float v0 = lo(raw[t]), v1 = hi(raw[t]);
-            mn0 = fminf(mn0, v0); mx0 = fmaxf(mx0, v0);
-            mn1 = fminf(mn1, v1); mx1 = fmaxf(mx1, v1);
+        for (int t = 1; t < KVC_WAVE; t++) {
+            const kvc_half2 x = __builtin_bit_cast(kvc_half2, raw[t]);
+            mn = __builtin_elementwise_min(mn, x);
+            mx = __builtin_elementwise_max(mx, x);
         }
-        g0 = kvc_group_params(mn0, mx0, a.eb);
-        g1 = kvc_group_params(mn1, mx1, a.eb);
+        const uint32_t mnw = __builtin_bit_cast(uint32_t, mn), mxw = __builtin_bit_cast(uint32_t, mx);
+        g0 = kvc_group_params(kvc_half_lo(mnw), kvc_half_lo(mxw), a.eb);
+        g1 = kvc_group_params(kvc_half_hi(mnw), kvc_half_hi(mxw), a.eb);
         const int8_t m0 = (int8_t)(int)g0.min_i, m1 = (int8_t)(int)g1.min_i;     // quantize with the minimum as it is stored
         g0.min_i = (float)m0;
         g1.min_i = (float)m1;
@@ -560,11 +554,12 @@ __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t 
     } else {                                             // one pair per 64-token block (kernels.cu:771-772)
         g0 = g1 = kvc_stored_params(a, row);
     }
+    const KvcPackedParams pp = kvc_packed_params(g0, g1);
     if (act) {
 #pragma unroll
         for (int t = 0; t < KVC_WAVE; t++) {
-            const uint32_t s2 = (uint32_t)kvc_quant_one(lo(raw[t]), g0) | ((uint32_t)kvc_quant_one(hi(raw[t]), g1) << 8);
-            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)s2;
+            const uint32_t u = kvc_quant_pair_biased(raw[t], pp);
+            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -581,7 +576,7 @@ __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t 
 // then reads channel c's vector.  Group parameters are per token (KVC_MASK_V_TOKEN) or per (token, batch
 // entry) (KVC_MASK_SIM_TOKEN; the tile lies inside one batch entry); the wave first stages its 128 triples
 // {scale, 1 / scale, min} in LDS.
-__device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, float *s_par,
+__device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t *s_par,
                                             uint32_t (&v)[32])
 {
     const int64_t stride = a.e.stride;
@@ -595,9 +590,8 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
         const int t = lane + 64 * k;
         const int64_t tk = row * KVC_V_TOKENS + t;
         const KvcGroupParams g = kvc_stored_params(a, a.mask == KVC_MASK_V_TOKEN ? tk : tk * a.B + b);
-        s_par[4 * t] = g.scale;
-        s_par[4 * t + 1] = g.rcp;
-        s_par[4 * t + 2] = g.min_i;
+        const KvcPackedParams pp = kvc_packed_params(g, g);          // the token's constants in both halves
+        *reinterpret_cast<uint4 *>(s_par + 4 * t) = make_uint4(pp.P2, pp.S2, pp.r2, pp.c2);
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -605,21 +599,17 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
     const __half *p = a.x + (row * KVC_V_TOKENS + 64 * half) * stride + ch;
 #pragma unroll 2
     for (int jj = 0; jj < 16; jj++) {
-        uint32_t w0 = 0, w1 = 0;
+        uint32_t u[4];
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int t = 64 * half + 4 * jj + k;
-            const uint32_t raw = *reinterpret_cast<const uint32_t *>(p + (int64_t)(4 * jj + k) * stride);
-            KvcGroupParams g;
-            g.scale = s_par[4 * t];
-            g.rcp = s_par[4 * t + 1];
-            g.min_i = s_par[4 * t + 2];
-            g.min_h = __float2half_rn(g.min_i);
-            const float v0 = __half2float(__ushort_as_half((unsigned short)(raw & 0xffffu)));
-            const float v1 = __half2float(__ushort_as_half((unsigned short)(raw >> 16)));
-            w0 |= (uint32_t)kvc_quant_one(v0, g) << (8 * k);
-            w1 |= (uint32_t)kvc_quant_one(v1, g) << (8 * k);
+            const uint4 c = *reinterpret_cast<const uint4 *>(s_par + 4 * t);
+            const KvcPackedParams pp = {c.x, c.y, c.z, c.w};
+            u[k] = kvc_quant_pair_biased(*reinterpret_cast<const uint32_t *>(p + (int64_t)(4 * jj + k) * stride), pp);
         }
+        // a01 = {channel 2 pr, 2 pr + 1 of token 4 jj | the same of token 4 jj + 1}; then four tokens of each channel
+        const uint32_t a01 = kvc_low_bytes4(u[0], u[1]), a23 = kvc_low_bytes4(u[2], u[3]);
+        const uint32_t w0 = kvc_low_bytes4(a01, a23), w1 = __builtin_amdgcn_perm(a23, a01, 0x07050301u);
         *reinterpret_cast<uint32_t *>(s_sym + (2 * pr) * RS + 64 * half + 4 * jj) = w0;
         *reinterpret_cast<uint32_t *>(s_sym + (2 * pr + 1) * RS + 64 * half + 4 * jj) = w1;
     }
@@ -636,7 +626,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
     __shared__ uint8_t s_len[KVC_WAVES_PER_WG][256];
     __shared__ uint32_t s_err, s_longest;
     __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];
-    __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];   // V: {scale, 1 / scale, min, -} per token
+    __shared__ __align__(16) uint32_t s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];   // V: the packed constants of every token
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid == 0) { s_err = 0; s_longest = 0; }
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
@@ -659,7 +649,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
 {
     __shared__ uint2 s_table[KVC_WAVES_PER_WG][256];
     __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];   // symbols first, then the payload image
-    __shared__ float s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];
+    __shared__ __align__(16) uint32_t s_par[IS_K ? 1 : KVC_WAVES_PER_WG][IS_K ? 4 : 4 * KVC_V_TOKENS];
     __shared__ uint32_t s_short[KVC_WAVES_PER_WG];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int64_t tile = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave;
@@ -671,7 +661,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     if (!p.ok) return;                                 // wave-uniform; nothing below involves another wave
     uint32_t *image = reinterpret_cast<uint32_t *>(s_sym[wave]);
     uint32_t v[32];
-    if (IS_K) kvc_front_k<false>(a, tile, lane, s_sym[wave], v);
+    if (IS_K) kvc_front_k(a, tile, lane, s_sym[wave], v);
     else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
     kvc_wave_lds_sync();                               // every lane holds its vector: the tile can be overwritten
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
@@ -680,6 +670,383 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     kvc_pack_vector(a.e, kvc_stream_start(a.e, tile, lane), v, s_table[wave], image, p.head, s_short[wave] != 0u);
     kvc_wave_lds_sync();
     kvc_write_image(a.e, p, lane, image);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// one pass: count, place and emit a tile in the same wave
+// ---------------------------------------------------------------------------------------------------
+// The two-pass encoder reads (and, in the fused store, quantizes) every tile twice and looks every symbol up twice,
+// because a tile's position in the payload is the sum of the sizes of all tiles before it.  Here a wave keeps its tile:
+// it looks its symbols up once (four codes of at most 8 bits joined into one group, the groups kept in the registers
+// that held the symbols), publishes the tile's size, finds its offset by looking back over the tiles before it
+// (decoupled look-back), and packs and writes the payload.  The offsets are the same exact prefix sums in tile order,
+// so the output is byte for byte that of the two-pass encoder.
+//
+// Two levels of status words.  A tile's is its own block_info, read and written as one 64-bit word
+// {u32 offset; u16 byte_num; u16 state}: a launch before this one marks every tile KVC_BI_NOT_READY, a wave that
+// knows its size writes {0, byte_num, KVC_BI_SIZE}, and once it knows its offset the final {offset, byte_num, 0}
+// (the reference's layout, state = padding = 0).  Runs of 64 consecutive tiles form a group with a word
+// {u32 bytes; u32 state} in the call's scratch slot: the wave of a group's last tile adds up the group
+// (KVC_BI_SIZE) and, once it knows what lies in front of the group, publishes the bytes up to the group's end
+// (state 0).  So a wave reads the sizes of the tiles before it in its own group (one 64-lane look), then walks the
+// group words backwards, 64 per look, adding sizes until a group with a known end stops the walk; tiles in flight
+// span a few dozen groups, so that is one or two looks.  Words that are not ready are polled again.
+// Progress: tiles are handed to workgroups in launch order, a wave publishes its size before it waits for anything,
+// and a group's size only needs the sizes of its own tiles, so whatever a wave waits for is published by waves that
+// started no later than itself and wait for nothing before publishing.  A wave that has polled KVC_LOOKBACK_POLLS
+// times gives up, flags the call (KVC_ENC_ERR_ORDER) and publishes what it has, so that every wave ends.
+constexpr uint32_t KVC_BI_SIZE = 1u, KVC_BI_NOT_READY = 0xffffu;
+constexpr uint32_t KVC_ENC_ERR_ORDER = 16u;         // a tile waited too long for the tiles before it
+constexpr uint32_t KVC_NO_CODE_LEN = 0x4000u;       // length of a symbol without a code: shows in any sum of lengths
+constexpr int KVC_LOOKBACK_POLLS = 1 << 18;         // some tenths of a second
+// The scratch slot of a one-pass call, in 32-bit words.  Tens of thousands of waves read the first tile's offset and
+// thousands of workgroups report maxima: on one cache line those accesses queue up behind each other (measured:
+// 0.5 ms of a 1.1 ms launch), so the offset gets a line that nothing is written to while the kernel runs, and the
+// maxima go to one of 32 lines picked by the workgroup number (kvc_encode_finish_kernel joins them afterwards).
+constexpr int KVC_ONCE_BASE_WORD = 32;               // copy of status[KVC_ENC_ST_BASE]
+constexpr int KVC_ONCE_PART_WORD = 64, KVC_ONCE_PART_LINES = 32, KVC_ONCE_PART_STRIDE = 32;   // {error bits, largest tile, longest stream}
+constexpr int KVC_ONCE_GROUP_WORD = KVC_ONCE_PART_WORD + KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE;
+constexpr int KVC_ONCE_MAX_GROUPS = (int)((KVC_WS_SLOT_BYTES - KVC_ONCE_GROUP_WORD * 4) / 8);
+
+__device__ __forceinline__ uint64_t kvc_bi_word(uint32_t offset, uint32_t byte_num, uint32_t state)
+{
+    return (uint64_t)offset | ((uint64_t)(byte_num & 0xffffu) << 32) | ((uint64_t)state << 48);
+}
+__device__ __forceinline__ uint64_t kvc_group_word(uint32_t bytes, uint32_t state) { return (uint64_t)bytes | ((uint64_t)state << 32); }
+__device__ __forceinline__ uint64_t *kvc_group_words(const KvcEncodeArgs &a)
+{
+    return reinterpret_cast<uint64_t *>(a.status + KVC_ONCE_GROUP_WORD);
+}
+__device__ __forceinline__ uint64_t kvc_status_load(const uint64_t *p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void kvc_status_store(uint64_t *p, uint64_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+
+__device__ __forceinline__ uint32_t kvc_wave_sum_u32(uint32_t v)
+{
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += (uint32_t)__shfl_xor((int)v, o, 64);
+    return v;
+}
+
+__global__ void __launch_bounds__(KVC_WG) kvc_encode_mark_kernel(KvcEncodeArgs a)
+{
+    const int64_t tile = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
+    if (tile < a.tiles) reinterpret_cast<uint64_t *>(a.block_infos)[tile] = kvc_bi_word(0u, 0u, KVC_BI_NOT_READY);
+    if (tile < (a.tiles + KVC_WAVE - 1) / KVC_WAVE) kvc_group_words(a)[tile] = kvc_group_word(0u, KVC_BI_NOT_READY);
+    if (blockIdx.x == 0) {
+        for (int i = threadIdx.x; i < KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE; i += KVC_WG) a.status[KVC_ONCE_PART_WORD + i] = 0u;
+        if (threadIdx.x == 0) a.status[KVC_ONCE_BASE_WORD] = a.status[KVC_ENC_ST_BASE];
+    }
+}
+
+// After the one-pass kernel: joins what the workgroups reported on their 32 lines into the call's status words.
+__global__ void __launch_bounds__(KVC_WAVE) kvc_encode_finish_kernel(KvcEncodeArgs a)
+{
+    const int lane = threadIdx.x;
+    uint32_t err = 0, tile = 0, stream = 0;
+    if (lane < KVC_ONCE_PART_LINES) {
+        const uint32_t *p = a.status + KVC_ONCE_PART_WORD + lane * KVC_ONCE_PART_STRIDE;
+        err = p[0];
+        tile = p[1];
+        stream = p[2];
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        err |= (uint32_t)__shfl_xor((int)err, o, 64);
+        const uint32_t t = (uint32_t)__shfl_xor((int)tile, o, 64), st = (uint32_t)__shfl_xor((int)stream, o, 64);
+        tile = t > tile ? t : tile;
+        stream = st > stream ? st : stream;
+    }
+    if (lane == 0) {
+        a.status[1] |= err;
+        a.status[2] = tile;
+        a.status[3] = stream;
+    }
+}
+
+// What a wave asks for as soon as it has published its size, and looks at only after it has packed its payload: the
+// words of the tiles before it in its group and of the 64 groups before its own.  The two round trips then run
+// while the wave works, and by the time it looks the words are usually final.
+struct KvcFirstLooks {
+    uint64_t tile_word, group_word;
+};
+
+__device__ __forceinline__ KvcFirstLooks kvc_look_back_ask(const KvcEncodeArgs &a, int64_t tile, int lane)
+{
+    const uint64_t *bi64 = reinterpret_cast<const uint64_t *>(a.block_infos);
+    const int64_t group = tile >> 6;
+    const int r = (int)(tile & 63);
+    KvcFirstLooks f;
+    f.tile_word = lane < r ? kvc_status_load(bi64 + (group << 6) + lane) : 0ull;
+    f.group_word = group - 1 - lane >= 0 ? kvc_status_load(kvc_group_words(a) + group - 1 - lane) : kvc_group_word(0u, 0u);
+    return f;
+}
+
+// First half of the look-back: the payload bytes of the tiles before `tile` in its own group; the wave of a group's last
+// tile then publishes the group's size.  *polls counts the looks that found a word not ready (wave-uniform).
+__device__ __forceinline__ uint32_t kvc_look_back_in_group(const KvcEncodeArgs &a, int64_t tile, uint32_t bn, int lane, uint64_t first_look,
+                                                           int *polls)
+{
+    const uint64_t *bi64 = reinterpret_cast<const uint64_t *>(a.block_infos);
+    const int64_t group = tile >> 6;
+    const int r = (int)(tile & 63);
+    uint32_t in_group = 0;
+    uint64_t w = first_look;
+    while (r > 0) {
+        if (!__any((uint32_t)(w >> 48) == KVC_BI_NOT_READY)) {
+            in_group = kvc_wave_sum_u32(lane < r ? (uint32_t)(w >> 32) & 0xffffu : 0u);
+            break;
+        }
+        if (++*polls > KVC_LOOKBACK_POLLS) break;
+        __builtin_amdgcn_s_sleep(2);
+        w = lane < r ? kvc_status_load(bi64 + (group << 6) + lane) : 0ull;
+    }
+    if ((r == 63 || tile == a.tiles - 1) && lane == 0)     // this wave speaks for its group
+        kvc_status_store(kvc_group_words(a) + group, kvc_group_word(in_group + bn, KVC_BI_SIZE));
+    return in_group;
+}
+
+// Second half: the payload bytes of the groups before the tile's own; the wave of a group's last tile then publishes
+// the bytes up to the end of its group.
+__device__ __forceinline__ uint32_t kvc_look_back_groups(const KvcEncodeArgs &a, int64_t tile, uint32_t in_group_and_own, int lane,
+                                                         uint64_t first_look, int *polls)
+{
+    uint64_t *groups = kvc_group_words(a);
+    const int64_t group = tile >> 6;
+    uint32_t before = 0;
+    int64_t j = group - 1;                                 // nearest group not yet accounted for
+    uint64_t w = first_look;                               // taken at j = group - 1
+    while (j >= 0 && *polls <= KVC_LOOKBACK_POLLS) {
+        const uint32_t state = (uint32_t)(w >> 32), bytes = (uint32_t)w;
+        const uint64_t not_ready = __ballot(state == KVC_BI_NOT_READY), known = __ballot(state == 0u);
+        const int first_nr = not_ready ? __builtin_ctzll(not_ready) : 64, first_kn = known ? __builtin_ctzll(known) : 64;
+        const int stop = first_kn < first_nr ? first_kn + 1 : first_nr;     // lanes below it count: sizes, then maybe an end
+        before += kvc_wave_sum_u32(lane < stop ? bytes : 0u);
+        if (first_kn < first_nr) break;                    // a group whose end is known closes the sum
+        j -= stop;
+        if (first_nr < 64) {
+            ++*polls;
+            __builtin_amdgcn_s_sleep(2);
+        }
+        const int64_t idx = j - lane;
+        w = idx >= 0 ? kvc_status_load(groups + idx) : kvc_group_word(0u, 0u);   // in front of the first group: nothing, and known
+    }
+    if (((tile & 63) == 63 || tile == a.tiles - 1) && lane == 0)
+        kvc_status_store(groups + group, kvc_group_word(before + in_group_and_own, 0u));
+    return before;
+}
+
+// A wave's (or the workgroup's) copy of the encode table for the one-pass kernel: as kvc_load_code_table, but an
+// entry without a usable code gets the length KVC_NO_CODE_LEN.
+__device__ __forceinline__ void kvc_load_code_table_marked(const KvcEncodeArgs &a, int64_t tile, uint2 *s_table, uint32_t *s_short, int lane)
+{
+    const uint2 *t = reinterpret_cast<const uint2 *>(kvc_table_of_row(a, tile / a.cols));
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const int i = lane + KVC_WAVE * k;
+        uint2 e = i < a.table_entries ? t[i] : make_uint2(0u, 0u);
+        if (e.y == 0u || e.y > 32u) e = make_uint2(0u, KVC_NO_CODE_LEN);
+        else if (e.y < 32u) e.x &= (1u << e.y) - 1u;      // nothing above the code's own bits
+        s_table[i] = e;
+        if (e.y > 8u && e.y != KVC_NO_CODE_LEN) atomicAnd(s_short, 0u);
+    }
+}
+
+// A tile whose payload is packed (in the wave's second LDS area) but not yet placed; the words its look-back reads
+// were asked for when its size was published.
+// payloads up to this size wait in LDS; larger tiles are placed at once (a V tile has half the symbols of a K tile of
+// head_dim 128 and needs LDS for its tokens' constants)
+constexpr int kvc_once_keep_bytes(int front) { return front == 2 ? 2048 : 4096; }
+struct KvcOncePending {
+    int64_t tile;                                          // -1: nothing pending
+    uint32_t bn, in_group;
+    bool in_group_known, packs;
+    KvcFirstLooks looks;
+};
+
+// Look back for a tile whose size has been published, publish its block_info and write its payload from the LDS
+// image (which starts on a word; the payload lands p.head bytes into an aligned word).  Returns error bits.
+__device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const KvcOncePending &pd, const uint32_t *image, uint32_t base,
+                                                   int lane, int *polls)
+{
+    const int64_t tile = pd.tile;
+    const uint32_t bn = pd.bn;
+    uint32_t in_group = pd.in_group;
+    if (!pd.in_group_known) in_group = kvc_look_back_in_group(a, tile, bn, lane, pd.looks.tile_word, polls);
+    const uint32_t off = base + in_group + kvc_look_back_groups(a, tile, in_group + bn, lane, pd.looks.group_word, polls);
+    uint32_t err = 0;
+    const bool gave_up = *polls > KVC_LOOKBACK_POLLS;
+    if (lane == 0) kvc_status_store(reinterpret_cast<uint64_t *>(a.block_infos) + tile, kvc_bi_word(off, bn, 0u));
+    if (gave_up) err |= KVC_ENC_ERR_ORDER;
+    KvcEmitPlace p;
+    p.off = off - a.base_global_offset;
+    p.bn = bn;
+    p.ok = !gave_up && pd.packs && (int64_t)p.off + bn <= a.encoded_cap;
+    p.head = p.ok ? (uint32_t)((reinterpret_cast<uintptr_t>(a.encoded) + p.off) & 3u) : 0u;
+    if (tile == a.tiles - 1 && lane == 0) {                // the call's totals, by the wave of the last tile
+        const uint32_t total = off + bn - base;
+        a.status[0] = total;
+        if ((int64_t)(base - a.base_global_offset) + total > a.encoded_cap) err |= KVC_ENC_ERR_CAPACITY;
+        if (a.idx_offset) {
+            a.idx_offset[0] = (uint32_t)a.tiles;
+            a.idx_offset[1] = total;
+        }
+    }
+    if (p.ok) kvc_write_image_shifted(a, p, lane, image);
+    return err;
+}
+
+// FRONT 0: uint8 symbols in; 1: fp16 K tile (quantized here); 2: fp16 V tile.
+// A wave works through `run` (one or two) consecutive tiles.  For each it counts (symbols -> codes and lengths, thread_infos),
+// publishes the size and asks for the words its look-back will read; then it places the tile before this one (look
+// back, block_info, payload out of the wave's second LDS area to its byte position) and packs this tile's payload
+// into that area, as an image that starts on a word (where the payload goes is not needed for that).  So a tile is
+// placed one tile's count after its size was published, when the tiles before it have published theirs: with the
+// look-back right behind the count, a tile waits 10 us on average for the slowest of the thousands of tiles in flight
+// before it (measured), as long as the rest of its work takes.
+// Dynamic LDS: the encode table (one for the workgroup, or one per wave when tile rows have codebooks of their own:
+// then run = 1), then per wave the tile of symbols, for V the tokens' constants, and the kept payload image.
+template <int FRONT>
+__global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs a, int run)
+{
+    extern __shared__ __align__(16) uint8_t s_dyn[];
+    __shared__ uint32_t s_short[KVC_WAVES_PER_WG], s_err, s_max_tile, s_longest;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const bool own_table = a.e.rows_per_codebook != 0;
+    uint2 *s_table = reinterpret_cast<uint2 *>(s_dyn) + (own_table ? wave * 256 : 0);
+    uint8_t *per_wave = s_dyn + (own_table ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2);
+    constexpr int PAR_BYTES = FRONT == 2 ? 4 * KVC_V_TOKENS * 4 : 0;
+    constexpr int KEEP_BYTES = kvc_once_keep_bytes(FRONT);
+    uint8_t *s_sym = per_wave + wave * (KVC_SYM_TILE_BYTES + PAR_BYTES + KEEP_BYTES + 16);
+    uint32_t *s_par = reinterpret_cast<uint32_t *>(s_sym + KVC_SYM_TILE_BYTES);
+    uint32_t *kept = reinterpret_cast<uint32_t *>(s_sym + KVC_SYM_TILE_BYTES + PAR_BYTES);
+    const int64_t tile0 = ((int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave) * run;
+    uint32_t *my_short = &s_short[own_table ? wave : 0];
+    if (tid == 0) { s_err = 0; s_max_tile = 0; s_longest = 0; }
+    if (lane == 0) s_short[wave] = 1u;
+    __syncthreads();
+    if (own_table ? tile0 < a.e.tiles : wave == 0) kvc_load_code_table_marked(a.e, tile0 < a.e.tiles ? tile0 : 0, s_table, my_short, lane);
+    __syncthreads();
+    const bool short_codes = *my_short != 0u;              // wave-uniform
+    const int nd = a.e.vec_len >> 2;
+    uint64_t *bi64 = reinterpret_cast<uint64_t *>(a.e.block_infos);
+    const uint32_t base = a.e.status[KVC_ONCE_BASE_WORD];
+    uint32_t err = 0, max_tile = 0, longest = 0;
+    int polls = 0;
+    KvcOncePending pd;
+    pd.tile = -1;
+#pragma unroll 1
+    for (int it = 0; it < run; it++) {
+        const int64_t tile = tile0 + it;
+        if (tile >= a.e.tiles) break;
+        uint32_t v[32];
+        if (FRONT == 1) kvc_front_k_once(a, tile, lane, s_sym, v);
+        else if (FRONT == 2) kvc_front_v(a, tile, lane, s_sym, s_par, v);
+        else kvc_load_vector(a.e, tile, lane, v);
+        kvc_wave_lds_sync();                               // every lane holds its vector: the tile area is free
+        uint32_t bits = 0;
+        uint32_t gl[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u}; // short codes: the four group lengths of registers 4 i .. 4 i + 3
+        if (short_codes) {
+#pragma unroll
+            for (int j = 0; j < 32; j++) {
+                if (j < nd) {
+                    const uint2 e0 = s_table[v[j] & 0xffu], e1 = s_table[(v[j] >> 8) & 0xffu];
+                    const uint2 e2 = s_table[(v[j] >> 16) & 0xffu], e3 = s_table[v[j] >> 24];
+                    const uint32_t len = e0.y + e1.y + e2.y + e3.y;
+                    // (the marked length of a symbol without a code shifts by nothing)
+                    v[j] = ((((e0.x << (e1.y & 31u)) | e1.x) << (e2.y & 31u) | e2.x) << (e3.y & 31u)) | e3.x;
+                    bits += len;
+                    gl[j >> 2] |= (len & 0xffu) << (8 * (j & 3));
+                }
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < 32; j++) {
+                if (j < nd) {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) bits += s_table[(v[j] >> (8 * k)) & 0xffu].y;
+                }
+            }
+        }
+        const bool bad = bits >= KVC_NO_CODE_LEN;          // a symbol without a code: the lane emits nothing
+        if (bad) bits = 0;
+        const uint32_t bytes = (bits + 7u) >> 3;
+        const uint32_t end = kvc_wave_inclusive_scan(bytes, lane);
+        a.e.thread_infos[tile * KVC_WAVE + lane] = (uint16_t)((end << 3) + (bytes << 3) - bits);
+        const uint32_t start = end - bytes;
+        const uint32_t tile_bytes = (uint32_t)__builtin_amdgcn_readlane((int)end, KVC_WAVE - 1);
+        const uint32_t bn = tile_bytes > 0xffffu ? 0xffffu : tile_bytes;
+        if (__any(bad)) err |= KVC_ENC_ERR_NO_CODE;
+        if (tile_bytes > (uint32_t)KVC_MAX_TILE_BYTES) err |= KVC_ENC_ERR_TILE_TOO_BIG;
+        const uint32_t lg = kvc_wave_max_dpp(bytes);
+        longest = lg > longest ? lg : longest;
+        max_tile = bn > max_tile ? bn : max_tile;
+        if (lane == 0) kvc_status_store(bi64 + tile, kvc_bi_word(0u, bn, KVC_BI_SIZE));
+        KvcOncePending cur;
+        cur.tile = tile;
+        cur.bn = bn;
+        cur.looks = kvc_look_back_ask(a.e, tile, lane);
+        // the wave that speaks for a group must not sit on the group's size (the groups after it wait for that word,
+        // and so would, one after the other, the waves that speak for them): it adds up its group at once
+        cur.in_group_known = (tile & 63) == 63 || tile == a.e.tiles - 1;
+        cur.in_group = 0;
+        if (cur.in_group_known) cur.in_group = kvc_look_back_in_group(a.e, tile, bn, lane, cur.looks.tile_word, &polls);
+        cur.packs = bn <= (uint32_t)KVC_MAX_TILE_BYTES;
+        // the tile before this one: its words have had this tile's count to arrive
+        if (pd.tile >= 0) {
+            err |= kvc_once_place(a.e, pd, kept, base, lane, &polls);
+            kvc_wave_lds_sync();                           // the kept image is read
+        }
+        pd.tile = -1;
+        const bool keep = bn <= (uint32_t)KEEP_BYTES && it + 1 < run && tile + 1 < a.e.tiles;
+        uint32_t *image = keep ? kept : reinterpret_cast<uint32_t *>(s_sym);
+        if (cur.packs) {
+            const uint32_t image_words = (bn + 3u) / 4u + 1u;
+            for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
+            kvc_wave_lds_sync();
+            if (short_codes) {
+                const uint32_t bitpos = start * 8u;
+                uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
+                uint64_t acc = 0;
+                if (!bad) {
+#pragma unroll
+                    for (int j = 0; j < 32; j++) {
+                        if (j < nd) {
+                            const uint32_t len = (gl[j >> 2] >> (8 * (j & 3))) & 0xffu;
+                            acc = (acc << len) | v[j];
+                            nacc += len;
+                            if (nacc >= 32u) {
+                                nacc -= 32u;
+                                if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
+                                w++;
+                            }
+                        }
+                    }
+                    if (nacc > 0 && w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
+                }
+            } else if (!bad) {
+                kvc_pack_vector(a.e, start, v, s_table, image, 0u, false);
+            }
+            kvc_wave_lds_sync();
+        }
+        if (keep) {
+            pd = cur;                                      // placed after the next tile is counted
+        } else {
+            err |= kvc_once_place(a.e, cur, image, base, lane, &polls);      // the wave's last tile, or too large to keep
+            kvc_wave_lds_sync();                           // the image is read: the area may take the next tile
+        }
+    }
+    if (lane == 0 && tile0 < a.e.tiles) {
+        if (err) atomicOr(&s_err, err);
+        atomicMax(&s_max_tile, max_tile);
+        atomicMax(&s_longest, longest);
+    }
+    __syncthreads();
+    if (tid == 0) {                                        // to this workgroup's line of the slot
+        uint32_t *part = a.e.status + KVC_ONCE_PART_WORD + (blockIdx.x % KVC_ONCE_PART_LINES) * KVC_ONCE_PART_STRIDE;
+        if (s_err) atomicOr(&part[0], s_err);
+        atomicMax(&part[1], s_max_tile);
+        atomicMax(&part[2], s_longest);
+    }
 }
 
 // What the fused path adds to an encode call: the fp16 source and how to quantize it.
@@ -715,6 +1082,7 @@ static int kvc_encode_errors(uint32_t bits, uint32_t total, int64_t encoded_cap)
         return kvc_fail(-3, "a tile encodes to more than %d bytes, which thread_info (u16) cannot address", KVC_MAX_TILE_BYTES);
     if (bits & KVC_ENC_ERR_CAPACITY)
         return kvc_fail(-3, "payload (%u bytes) does not fit the encoded_data buffer (%lld bytes)", total, (long long)encoded_cap);
+    if (bits & KVC_ENC_ERR_ORDER) return kvc_fail(-3, "one-pass encoder: a tile waited too long for the tiles before it");
     return 0;
 }
 
@@ -767,7 +1135,7 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     const unsigned wgs = (unsigned)((a.tiles + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
     const KvcStoreSource *src = c.src;
     const int is_k = c.is_k;
-    KvcStoreArgs sa;
+    KvcStoreArgs sa = {};
     if (src) {
         sa.e = a;
         sa.x = reinterpret_cast<const __half *>(src->x_f16);
@@ -780,6 +1148,31 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
         sa.scale_f16 = reinterpret_cast<__half *>(src->scale_f16);
     }
     hipLaunchKernelGGL(kvc_encode_init_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
+    // one pass (each wave counts, places and emits its tile) where the block_infos can serve as 64-bit status words
+    if (kvc_option(KVC_OPT_ENCODE_ONE_PASS) != 0 && ((uintptr_t)c.d_block_infos & 7) == 0 &&
+        (a.tiles + KVC_WAVE - 1) / KVC_WAVE <= KVC_ONCE_MAX_GROUPS) {
+        if (!src) sa.e = a;
+        const int front = !src ? 0 : is_k ? 1 : 2;
+        const size_t lds = (size_t)(a.rows_per_codebook ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2) +
+                           (size_t)KVC_WAVES_PER_WG * (KVC_SYM_TILE_BYTES + (front == 2 ? 4 * KVC_V_TOKENS * 4 : 0) + kvc_once_keep_bytes(front) + 16);
+        hipLaunchKernelGGL(kvc_encode_mark_kernel, dim3((unsigned)((a.tiles + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a);
+        // two tiles per wave (the look-back of the first hides behind the count of the second) where all tiles share
+        // the codebook and there are enough of them to keep the chip full.  Longer runs would chain the groups: a wave
+        // would place a tile (which needs the sizes of all groups before it) before it counts and publishes a later one.
+        const int want = kvc_option(KVC_OPT_ENCODE_ONE_PASS);
+        int run = want == 1 ? (a.tiles >= 8192 ? 2 : 1) : want - 1;       // 2, 3: always one, two tiles per wave
+        run = run < 1 ? 1 : run > 2 ? 2 : run;
+        if (a.rows_per_codebook != 0) run = 1;
+        const unsigned wgs1 = (unsigned)((a.tiles + (int64_t)run * KVC_WAVES_PER_WG - 1) / ((int64_t)run * KVC_WAVES_PER_WG));
+        if (front == 0) hipLaunchKernelGGL(kvc_encode_once_kernel<0>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+        else if (front == 1) hipLaunchKernelGGL(kvc_encode_once_kernel<1>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+        else hipLaunchKernelGGL(kvc_encode_once_kernel<2>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+        hipLaunchKernelGGL(kvc_encode_finish_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
+        if (a.result || a.stream_bytes) hipLaunchKernelGGL(kvc_encode_publish_kernel, dim3(1), dim3(1), 0, stream, a);
+        KVC_HIP(hipGetLastError());
+        *slot_out = slot;
+        return 0;
+    }
     if (!src) hipLaunchKernelGGL(kvc_encode_count_kernel, dim3(wgs), dim3(KVC_WG), 0, stream, a);
     else if (is_k) hipLaunchKernelGGL(kvc_store_count_kernel<true>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);
     else hipLaunchKernelGGL(kvc_store_count_kernel<false>, dim3(wgs), dim3(KVC_WG), 0, stream, sa);

@@ -20,13 +20,24 @@ CASES = [  # is_k, mode, B, H, D, dist
     (False, "TokenQuant", 1, 4, 128, "gauss"),
     (False, "TokenQuant", 2, 4, 96, "laplace"),
     (False, "TokenQuant", 3, 2, 32, "gauss"),
+    # magnitudes far from 1: the packed fp16 quantizer rescales every group by a power of two
+    (True, "ChannelQuant", 1, 2, 128, "gauss_tiny"),
+    (True, "ChannelQuant", 2, 2, 96, "laplace_big"),
+    (True, "BlockQuant", 1, 2, 64, "gauss_big"),
+    (False, "TokenQuant", 2, 2, 96, "laplace_tiny"),
+    (False, "TokenQuant", 1, 4, 128, "gauss_big"),
 ]
 
 
 def _data(is_k, T, B, H, D, dist, seed):
+    dist, _, mag = dist.partition("_")
+    # exact power-of-two factors: group scales near 2^-12 (small normal and subnormal fp16 values) and near 2^7
+    factor = {"": 1.0, "tiny": 2.0 ** -12, "big": 2.0 ** 6}[mag]
     if dist == "laplace":
-        return S.synth_laplace(T, B, H, D, seed)
-    return (S.synth_k if is_k else S.synth_v)(T, B, H, D, seed)
+        x = S.synth_laplace(T, B, H, D, seed)
+    else:
+        x = (S.synth_k if is_k else S.synth_v)(T, B, H, D, seed)
+    return x if factor == 1.0 else (x.float() * factor).clamp(-60000.0, 60000.0).to(torch.float16)
 
 
 @pytest.mark.parametrize("is_k,mode,B,H,D,dist", CASES)
@@ -258,3 +269,44 @@ def test_unbuilt_codebook_flags_the_encode_on_the_device():
                    encoded=payload, result=result)
     with pytest.raises(KvcompError, match="codebook"):
         m.encode_result(result, payload.numel())
+
+
+@pytest.mark.parametrize("one_pass", [0, 2, 3])
+@pytest.mark.parametrize("is_k,D,dist", [(True, 96, "laplace"), (False, 128, "gauss"), (True, 128, "gauss_tiny")])
+def test_one_pass_and_two_pass_encoders_write_the_same_bytes(is_k, D, dist, one_pass):
+    """The tile encoder runs in one pass (waves look back over the sizes published by the tiles before them; one or
+    two tiles per wave) or in two (count, offsets, emit): payload, block_infos and thread_infos must not depend on
+    which, for the fused store and for the encoder that starts from symbols, over enough tiles (> 4096) that waves of
+    many workgroups wait for each other, and for a second store appended behind the first."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    T, B, H = 4096, 2, 16
+    eb = 0.1 if is_k else 0.2
+    x1, x2 = _data(is_k, T, B, H, D, dist, 21).to(DEV), _data(is_k, 512, B, H, D, dist, 22).to(DEV)
+    results = []
+    for mode in (1, one_pass):                       # the default first, then the variant under test
+        was = _lib.set_option("encode_one_pass", mode)
+        try:
+            fused, plain = KVCompCtx(is_k, B, H, D, eb), KVCompCtx(is_k, B, H, D, eb)
+            for ctx in (fused, plain):
+                ctx.build_codebook([x1[:512], x2])
+            fused.store(x1, want_symbols=False)
+            fused.store(x2, want_symbols=False)
+            plain.store(x1)
+            plain.store(x2)
+            results.append((fused, plain))
+        finally:
+            _lib.set_option("encode_one_pass", was)
+    (f1, p1), (f2, p2) = results
+    for name in ("quant_scales", "quant_min_ints", "thread_infos", "block_infos", "encoded_data"):
+        a = getattr(f1, name)
+        for other in (p1, f2, p2):
+            b = getattr(other, name)
+            assert a.shape == b.shape and torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
+    assert (f1.max_tile_bytes, f1.max_stream_bytes) == (f2.max_tile_bytes, f2.max_stream_bytes) == (p2.max_tile_bytes, p2.max_stream_bytes)
+    # and the oracle agrees with the first store's payload
+    o = O.quant(S.np16(S.blocked(x1.cpu(), f1.block_size)), _oracle_mask(f1), eb)
+    pay, bi, ti = O.encode_tiles(o[3], is_k, f1.encode_codebook.cpu().numpy(), 0, vec_len=D if is_k else 128)
+    assert np.array_equal(f1.encoded_data.cpu().numpy()[:pay.size], pay)
+    assert np.array_equal(f1.block_infos.cpu().numpy()[:bi.size], bi)
