@@ -84,11 +84,12 @@ int kvc_abi_version(void);
  *                           first 70 % of the tiles, 2 for the next 20 %, single tiles last; 0: never (every wave
  *                           takes "fused_tiles_per_wave" tiles of one tile row); r * 10000 + p * 100 + q: runs of r
  *                           for the first p %, r / 2 for the next q %, r / 4 and 1 for halves of the rest.
- *   "encode_one_pass":       1 (default): the tile encoders (kvc_k_/v_entropy_encode, kvc_store_fused, kvc_encode_async) read
- *                           their input once: a wave counts its tiles, finds their place in the payload by looking back
+ *   "encode_one_pass":       1 (default): the fused quantize + encode (kvc_store_fused, kvc_encode_async from fp16) reads
+ *                           its input once: a wave quantizes and counts its tiles, finds their place in the payload by looking back
  *                           over the sizes the tiles before it have published, and emits them; 0: two passes (count,
  *                           offsets, emit), also taken when block_infos is not 8-byte aligned or the call has more than
- *                           96 256 tiles; 2 / 3: one pass with always one / two tiles per wave.  Same bytes either way.
+ *                           96 256 tiles, and by the encoders that start from uint8 symbols; 2 / 3: one pass for every encoder, with
+ *                           always one / two tiles per wave.  Same bytes either way.
  *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
  *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile

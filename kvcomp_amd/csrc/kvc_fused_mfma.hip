@@ -428,17 +428,8 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     const uint32_t pbits = 2u * lmax;
     // two symbols per look-up: twice the longest code fits the index, and no symbol's fp16 pattern needs the five
     // bits the lengths of a two-symbol entry go to (header word 6: OR of all the patterns)
-#ifdef KVC_EXP_KIND
-    constexpr bool EXPF = KIND == KVC_EXP_KIND && REP == 1 && ROUNDED;
-#else
-    constexpr bool EXPF = false;
-#define KVC_EXP_PAIRS 0
-#define KVC_EXP_PER 12
-#define KVC_EXP_SKEW 0
-#endif
-    const bool pairs_rt = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
+    const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
                        (1u << pbits) <= (uint32_t)a.table_words && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
-    const bool pairs = EXPF ? (bool)KVC_EXP_PAIRS : pairs_rt;
     if (pairs) {
         // the one-symbol table goes to the (not yet used) per-wave areas; the two-symbol table is derived from it
         uint32_t *tmp = smem + a.table_words;
@@ -461,7 +452,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     const uint32_t mask4 = ((1u << lbits) - 1u) << 2, maskp = ((1u << pbits) - 1u) << 2;
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
     // symbols per refill in the main part (a multiple of four); what is left goes eight per refill
-    const int per = EXPF ? KVC_EXP_PER : pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
+    const int per = pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
     int n_main = (n / per) * per;
     while ((n - n_main) % 8 != 0) n_main -= per;
     const uint32_t fe = kvc_lds_addr(smem);                            // 0: the table opens the workgroup's LDS
@@ -529,8 +520,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                     if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                 }
             };
-            if (EXPF) run(std::integral_constant<bool, (bool)KVC_EXP_SKEW>{});
-            else if (a.skew) run(std::true_type{});
+            if (a.skew) run(std::true_type{});
             else run(std::false_type{});
             // register i of lane 4 b + j: row 4 b + i, column 4 set + j; the even columns take their low parts from
             // the lane to their right and carry the results of query head 2 set + j / 2
