@@ -76,6 +76,8 @@ int kvc_abi_version(void);
  *   "fused_mfma":           -1 (default) or 1: the multiply-accumulate of the fused matvecs runs on the matrix cores
  *                           (v_mfma_f32_4x4x4_16b_f16) wherever those kernels apply (codes of at most 7 bits, results
  *                           that can be stored four at a time); 0: never (fp32 multiply-adds on the vector units).
+ *   "fused_half_table":      1 (default): for codes of 6 or 7 bits the matrix-core kernels use two-byte decode table entries
+ *                           (64 entries = one LDS word per bank); 0: four-byte entries.
  *   "fused_builtin_dpp":     0 (default): the fp32-FMA kernels pick their operand out of a quad of lanes with a permute
  *                           written as inline assembly on the multiply-add itself; 1: through the compiler's lane-
  *                           permute intrinsic (same result bit for bit; a cross-check against toolchain changes).

@@ -857,6 +857,7 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
     a.out_words = 0;
     a.double_window = kvc_option(KVC_OPT_FUSED_DOUBLE_WINDOW);
     a.builtin_dpp = kvc_option(KVC_OPT_FUSED_BUILTIN_DPP) != 0;
+    a.half_table = kvc_option(KVC_OPT_FUSED_HALF_TABLE) != 0;
     if (allow_pairs && extra_words == 0 && max_code_bits >= 1 && 2 * max_code_bits <= pair_limit) {
         a.pair_bits = 2 * max_code_bits;
         // eight bytes per entry (fp32 symbols), four in the matrix-core kernels (fp16 symbols)

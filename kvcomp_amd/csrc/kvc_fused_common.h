@@ -34,6 +34,7 @@ struct KvcFusedArgs {
     int pair_bits;       // index width of the two-symbol table the host made room for; 0 = none
     int double_window;   // refill 64 stream bits at a time where the vector length allows
     int builtin_dpp;     // fp32-FMA kernels: lane permutes through the compiler's intrinsic instead of inline assembly
+    int half_table;      // matrix-core kernels: two-byte table entries for codes of 6 or 7 bits
     // kvc_expand_kernel (plain decode, decode + dequantize): no x; the operand table holds {scale, min} per element
     // Rounded mode of the matvec kernels: every (sym + min) * scale is rounded to fp16 before it meets q / p, as the
     // reference's dequantizer does (models/cache/kvcomp_encode.py:146); the operand table then holds
@@ -155,6 +156,7 @@ struct KvcVec {
 // LDS accessed by its byte offset: the table's offset is a multiple of its size, so "window bits | offset"
 // is the entry's address.
 typedef __attribute__((address_space(3))) uint32_t kvc_lds_u32;
+typedef __attribute__((address_space(3))) uint16_t kvc_lds_u16;
 
 // compile-time loop: body(std::integral_constant<int, 0>) ... body(std::integral_constant<int, N - 1>)
 template <int N, int I = 0, class Body>

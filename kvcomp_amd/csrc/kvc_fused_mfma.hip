@@ -224,27 +224,44 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
 // 2 G symbols per refill of 64 stream bits (G from each half window; 2 G a multiple of four), n a multiple of 2 G.
 // bptr: LDS byte address of this lane's column in the operand table of the group the loop starts with;
 // msptr: of that group's minima and scales (rounded mode).  Both advance with the groups consumed.
-template <int G, bool SKEW, int NM, bool ROUNDED, bool BCAST>
+// HALF: two-byte table entries {symbol as fp16 | code length in the bits that symbols below 64 leave clear}: a table of
+// 64 entries then fills 32 words, one per LDS bank, and two lanes that read different entries of one bank read the same
+// word, which the LDS serves in one cycle (with four-byte entries a 64-entry table has two words per bank and 42 % of
+// its LDS cycles are bank conflicts).  Costs an instruction per two symbols (join and mask instead of a byte permute);
+// the lengths of a half window (at most 4 x 7 bits) are summed in five bits, above which symbol bits pile up.
+template <int G, bool SKEW, int NM, bool ROUNDED, bool BCAST, bool HALF = false>
 __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32_t fe, uint32_t mask4, int n,
                                              uint32_t &bptr, uint32_t &msptr, kvc_f4 (&acc)[NM], bool holder)
 {
     static_assert((2 * G) % 4 == 0, "whole groups of four per refill");
+    static_assert(!HALF || G <= 4, "the lengths of a half window must fit five bits");
     asm volatile("" : "+v"(msptr));      // kept in a vector register: one add per round instead of a move per read
     for (int i = 0; i < n; i += 2 * G) {
         const kvc_lds_word *wp = (const kvc_lds_word *)(uintptr_t)kvc_refill_address<SKEW>(sbase, u);
         const uint32_t w0 = wp[0], w1 = wp[1], w2 = wp[2];
         const uint32_t lo = __builtin_amdgcn_alignbit(w1, w0, u), hi = __builtin_amdgcn_alignbit(w2, w1, u);
-        uint32_t R = lo, es = 0;
+        uint32_t R = lo, es = 0, used1 = 0;
         uint32_t e[2 * G];
         kvc_static_for<2 * G>([&](auto g_) {
             constexpr int g = decltype(g_)::value;
-            if (g == G) R = __builtin_amdgcn_alignbit(hi, lo, es);
-            e[g] = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fe);
+            if (g == G) {
+                R = __builtin_amdgcn_alignbit(hi, lo, es);       // (shifts by the low five bits of es)
+                if (HALF) used1 = es & 31u, es = 0;
+            }
+            if constexpr (HALF) e[g] = *(const kvc_lds_u16 *)(uintptr_t)((R & mask4) | fe);
+            else e[g] = *(const kvc_lds_u32 *)(uintptr_t)((R & mask4) | fe);
             if (g != G - 1 && g != 2 * G - 1) R = __builtin_amdgcn_alignbit(R, R, e[g]);
             es += e[g];
             if constexpr (g % 4 == 3) {
                 constexpr int q = g / 4;
-                uint32_t a01 = kvc_pack_hi16(e[g - 3], e[g - 2]), a23 = kvc_pack_hi16(e[g - 1], e[g]);
+                uint32_t a01, a23;
+                if constexpr (HALF) {
+                    a01 = ((e[g - 2] << 16) | e[g - 3]) & 0xffe0ffe0u;
+                    a23 = ((e[g] << 16) | e[g - 1]) & 0xffe0ffe0u;
+                } else {
+                    a01 = kvc_pack_hi16(e[g - 3], e[g - 2]);
+                    a23 = kvc_pack_hi16(e[g - 1], e[g]);
+                }
                 if (ROUNDED) {
                     const kvc_w4 ms = *(const kvc_lds_w4 *)(uintptr_t)(msptr + q * 16);
                     a01 = kvc_dequant_pair(a01, ms.x, ms.z);
@@ -255,7 +272,7 @@ __device__ __forceinline__ void kvc_mfma_dot(uint32_t sbase, uint32_t &u, uint32
                     acc[s] = kvc_mfma4<BCAST>(a01, a23, kvc_read_columns<BCAST>(bptr + (q * NM + s) * 32, holder), acc[s]);
             }
         });
-        u += es & 0xffu;
+        u += HALF ? used1 + (es & 31u) : es & 0xffu;
         bptr += (2 * G / 4) * NM * 32;
         msptr += (2 * G / 4) * 16;
     }
@@ -430,6 +447,9 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     // bits the lengths of a two-symbol entry go to (header word 6: OR of all the patterns)
     const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
                        (1u << pbits) <= (uint32_t)a.table_words && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
+    // codes of 6 or 7 bits: two-byte entries (see kvc_mfma_dot), where no symbol's fp16 pattern needs its five lowest bits
+    const bool half_table = fast_book && !pairs && lbits >= 6u && a.half_table != 0 && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
+    const uint32_t lead_bits = half_table ? 1u : 2u;                   // bits of the window below the table index
     if (pairs) {
         // the one-symbol table goes to the (not yet used) per-wave areas; the two-symbol table is derived from it
         uint32_t *tmp = smem + a.table_words;
@@ -442,6 +462,12 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             smem[idx] = (e1 & 0xffff0000u) | (e0 >> 16) | ((e0 & 0xffu) + (e1 & 0xffu));
         }
         __syncthreads();
+    } else if (half_table) {
+        uint16_t *t16 = reinterpret_cast<uint16_t *>(smem);
+        for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) {
+            const uint32_t e = fentry(i);
+            t16[i] = (uint16_t)((e >> 16) | (e & 0xffu));
+        }
     } else if (fast_book) {
         for (uint32_t i = tid; i < (1u << lbits); i += KVC_WG) smem[i] = fentry(i);
     }
@@ -449,7 +475,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     for (int i = lane; i < SLOTS * T::BTAB_SLOT_WORDS; i += KVC_WAVE) btab[i] = 0;
     if (lane < KVC_PACK_LEAD) pack[lane] = 0;
     __syncthreads();
-    const uint32_t mask4 = ((1u << lbits) - 1u) << 2, maskp = ((1u << pbits) - 1u) << 2;
+    const uint32_t mask4 = ((1u << lbits) - 1u) << lead_bits, maskp = ((1u << pbits) - 1u) << 2;
     const int n = IS_K ? D : KVC_V_TOKENS;                             // symbols per lane stream
     // symbols per refill in the main part (a multiple of four); what is left goes eight per refill
     const int per = pairs ? (pbits <= 7u ? 16 : 12) : (lmax <= 3u ? 16 : lmax <= 5u ? 12 : 8);
@@ -464,7 +490,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     int sel = 0;
     uint32_t first, longest;
     KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
-    if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;       // two bits before the lane's first code
+    if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;       // one or two bits before the lane's first code
     kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col, lane, raw, btab, mstab, bias, unscale, sel);
     kvc_wave_sync();
     for (int it = 0; it < ntiles; it++) {
@@ -517,7 +543,8 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                     if (per == 16) kvc_mfma_dot<8, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
                     else if (per == 12) kvc_mfma_dot<6, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
                     const int rest = per == 8 ? n : n - n_main;
-                    if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
+                    if (rest && half_table) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST, true>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
+                    else if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                 }
             };
             if (a.skew) run(std::true_type{});
@@ -553,7 +580,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
         } else {
             KvcVec<REP> res;
             if (st.fits)
-                res = kvc_mfma_slow_tile<REP, false, ROUNDED>(pack, (uint32_t)a.pack_logical, st.u0 + 2u, lut_g, n, my_btab,
+                res = kvc_mfma_slow_tile<REP, false, ROUNDED>(pack, (uint32_t)a.pack_logical, st.u0 + lead_bits, lut_g, n, my_btab,
                                                               my_mstab, (uint32_t)a.skew);
             else
                 res = kvc_mfma_slow_tile<REP, true, ROUNDED>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_btab, my_mstab, 0u);
@@ -571,7 +598,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             int lane_s = lane;
             asm volatile("" : "+v"(lane_s));
             st = kvc_stage_payload(a, lane_s, raw, pack, first, longest);
-            if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - 2u;
+            if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;
             kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row_next, col_next, lane_s, raw, btab, mstab, bias, unscale, sel);
             kvc_wave_sync();
         }
