@@ -243,6 +243,39 @@ def test_compressed_attention_under_every_staging_plan(rows, tiles_per_wave, D, 
     assert L.kvc_set_option(b"no_such_option", 1) != 0
 
 
+@pytest.mark.parametrize("schedule", [46030, 85035, 25040, 30000, 166020, 10000])
+@pytest.mark.parametrize("D,rep", [(128, 1), (96, 2)])
+def test_compressed_attention_under_every_tile_schedule(schedule, D, rep):
+    """The matrix-core kernels of a long stream walk the row-major tile sequence in segments, the waves of a segment
+    taking runs of 8, 4, 2 or 1 consecutive tiles (across tile rows, and cut short where a segment or the stream ends).
+    Forced here on a small cache whose tile counts are no multiple of any run: every schedule must give the output of
+    the plain launch bit for bit, in both arithmetic modes."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd.ctx import KVCompCtx
+    from kvcomp_amd.attention import CompressedAttention
+    _config(k_mode="ChannelQuant")
+    T, B, H = 7 * 128 + 31, 2, 3                      # K: 14 x 6 tiles; V: 7 rows of 12 (D 128) or 9 (D 96) tiles
+    k, v = S.synth_k(T, B, H, D).to(DEV), S.synth_v(T, B, H, D).to(DEV)
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(k)
+    vctx.store(v)
+    q = S.synth_q(B, H * rep, D).to(DEV)
+    for rounded in (1, 0):
+        saved = {n: _lib.set_option(n, v_) for n, v_ in (("fused_rounded", rounded), ("fused_schedule", 0))}
+        try:
+            plain = CompressedAttention(kctx, vctx).attend(q)
+            _lib.set_option("fused_schedule", schedule)
+            out = CompressedAttention(kctx, vctx).attend(q)
+        finally:
+            for n, v_ in saved.items():
+                _lib.set_option(n, v_)
+        assert torch.equal(out, plain)
+    kd, vd = kctx.get()[0].float(), vctx.get()[0].float()
+    s_ = torch.einsum("tbhd,bhd->bht", kd.repeat_interleave(rep, dim=2), q.float()) / D ** 0.5
+    ref = torch.einsum("tbhd,bht->bhd", vd.repeat_interleave(rep, dim=2), torch.softmax(s_, dim=-1))
+    assert (plain - ref).abs().max() <= 3e-3 * ref.abs().max()          # (the unrounded mode's result was the last)
+
+
 @pytest.mark.parametrize("D,rep,eb_k", [(128, 1, 0.1), (96, 2, 0.05), (64, 4, 0.3), (128, 8, 0.1)])
 def test_lane_permute_in_assembly_equals_the_compilers(D, rep, eb_k):
     """The fp32-FMA kernels fetch one of four operands from the lanes of a quad with a permute that rides on the
