@@ -219,7 +219,7 @@ def measured_traffic(workload, kernel):
     return t.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
-def run_decode_loop(args):
+def run_decode_loop(args, emit=True):
     """cfg4 without the model around it: every layer of a Llama-2-7B-shaped stack keeps a compressed K and V cache;
     a step appends one new token per sequence to every layer (compressing the 64- / 128-token blocks that leave
     the uncompressed tails) and runs decode attention over the whole cache of that layer.  Projections, MLPs and
@@ -286,7 +286,82 @@ def run_decode_loop(args):
                    "not_run": "projections, MLP, norms, sampling (outside this path)"},
         "roofline": None, "cpu_baseline": None,
     }
-    print(json.dumps(result), flush=True)
+    if emit:
+        print(json.dumps(result), flush=True)
+    del layers
+    torch.cuda.empty_cache()
+    return result
+
+
+def quick_attention(name, steps=50, warmup=10):
+    """One of the smaller configurations, measured the short way for the default run's `config.other_configs`: build the
+    compressed cache, check one result against fp32 attention over the dequantized cache, time `steps` decode-attention
+    passes (default arithmetic) over copies of the cache that together exceed the last-level cache."""
+    import copy
+    import torch
+    from kvcomp_amd.ctx import KVCompCtx, KVCompCacheConfig, KVCompCacheConfigStatic, QuantMode
+    from kvcomp_amd import attention as A
+    cfg = WORKLOADS[name]
+    dev = torch.device("cuda:0")
+    B, H, Hq, D, T = cfg["B"], cfg["H"], cfg["Hq"], cfg["D"], cfg["T"]
+    KVCompCacheConfigStatic.config = KVCompCacheConfig(name, QuantMode.ChannelQuant, QuantMode.TokenQuant, 64, 128, 64, 128,
+                                                       cfg["eb_k"], cfg["eb_v"])
+    k, v = make_kv(cfg, dev)
+    kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
+    kctx.store(k, want_symbols=False)
+    vctx.store(v, want_symbols=False)
+    del k, v
+    g = torch.Generator().manual_seed(1236)
+    q = torch.randn(B, Hq, D, generator=g, dtype=torch.float32).to(torch.float16).to(dev)
+    kb, vb = kctx.compressed_bytes(), vctx.compressed_bytes()
+    n = max(3, min(32, -(-600_000_000 // (kb + vb))))
+    attns = [A.CompressedAttention(kctx, vctx)] + [A.CompressedAttention(copy.deepcopy(kctx), copy.deepcopy(vctx)) for _ in range(n - 1)]
+    out = torch.empty(B, Hq, D, dtype=torch.float32, device=dev)
+    attns[0].attend(q, out=out)
+    rep = Hq // H
+    kd, vd = kctx.get_only_compressed()[0][:, 0, 0].float(), vctx.get_only_compressed()[0][:, 0, 0].float()   # batch 0, KV head 0
+    sc = torch.einsum("td,rd->rt", kd, q[0, :rep].float()) / D ** 0.5
+    ref = torch.einsum("td,rt->rd", vd, torch.softmax(sc, dim=-1))
+    err = float((out[0, :rep] - ref).abs().max() / ref.abs().max())
+    assert err <= 1e-3, "%s: attention differs from fp32 attention over the dequantized cache by %.2e" % (name, err)
+    for i in range(warmup):
+        attns[i % n].attend(q, out=out)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        attns[i % n].attend(q, out=out)
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) / steps * 1e3
+    k_ms = v_ms = 0.0
+    for i in range(steps):
+        kms = []
+        attns[i % n].attend(q, out=out, kernel_ms=kms)
+        k_ms += kms[0] / steps
+        v_ms += kms[1] / steps
+    res = {"workload": cfg["desc"], "ms_per_step": round(ms, 4), "GBs": round((kb + vb) / (ms * 1e-3) / 1e9, 1),
+           "pct_hbm_peak": round(100 * (kb + vb) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+           "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)}, "compressed_bytes": {"k": kb, "v": vb},
+           "compression_ratio": {"k": round(kctx.get_cr(), 3), "v": round(vctx.get_cr(), 3)},
+           "k_max_code_bits": kctx.max_code_bits, "v_max_code_bits": vctx.max_code_bits,
+           "cache_copies_cycled": n, "steps": steps, "check_max_error": err}
+    log("[bench] %s: step %.3f ms (%.0f GB/s of compressed bytes), fused K %.3f ms, fused V %.3f ms" % (name, ms, res["GBs"], k_ms, v_ms))
+    del attns, kctx, vctx
+    torch.cuda.empty_cache()
+    return res
+
+
+def other_configs(args):
+    """The configurations besides the default one, each measured briefly in the same process."""
+    import types
+    res = {}
+    for name in ("cfg2", "cfg3"):
+        res[name] = quick_attention(name)
+    loop = run_decode_loop(types.SimpleNamespace(steps=20, warmup=5, sync_store=False), emit=False)
+    res["cfg4_cache_loop"] = {"workload": loop["config"]["workload"], "ms_per_step": loop["ms_per_step"], "tokens_per_s": loop["value"],
+                              "steps": loop["steps"], "compression_ratio_whole_cache": loop["config"]["compression_ratio_whole_cache"],
+                              "prefill_compress_s": loop["config"]["prefill_compress_s"], "not_run": loop["config"]["not_run"]}
+    log("[bench] cfg4 cache loop: %.2f ms per step, %.0f tokens/s" % (loop["ms_per_step"], loop["value"]))
+    return res
 
 
 def run_model_decode(args):
@@ -375,6 +450,8 @@ def main():
     ap.add_argument("--no-sweep", action="store_true", help="cfg5: skip the sweep over K's error bound")
     ap.add_argument("--sync-store", action="store_true",
                     help="cfg4: wait for the device after every encode (the reference's behaviour) instead of queuing it")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="default workload: skip the short measurements of cfg2, cfg3 and the cfg4 cache loop (config.other_configs)")
     ap.add_argument("--no-graph", action="store_true", help="skip the replay of the step as a captured HIP graph")
     ap.add_argument("--model-layers", type=int, default=0,
                     help="cfg4 only: run the Llama-2-7B architecture itself (random weights) with this many layers (32 = "
@@ -608,6 +685,12 @@ def main():
         "roofline": {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": measured_traffic(args.workload, dom)},
     }
+    if args.workload == DEFAULT_WORKLOAD and args.eb_k is None and not args.no_other_configs:
+        attns = at = res = None                        # the copies of this cache are released first
+        torch.cuda.empty_cache()
+        static = KVCompCacheConfigStatic.config
+        result["config"]["other_configs"] = other_configs(args)
+        KVCompCacheConfigStatic.config = static
     if not args.no_cpu_baseline:
         log("[bench] timing the CPU restatement of the reference's path ...")
         k_head = make_kv(dict(cfg, T=min(T, 2048)), torch.device("cpu"))[0]
