@@ -5,7 +5,9 @@
 Objects are compiled in parallel (one hipcc process per source file) and linked into one shared
 library that exports the C ABI declared in include/kvcomp_hip.h.
 """
+import json
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -22,7 +24,11 @@ FLAGS = [
     # packed-fp32 VALU forms are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
+    # the code generator's own account of every kernel (registers, spills, scratch, LDS), kept beside the objects
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+RESOURCES = os.path.join(HERE, "build", "kernel_resources.json")
+_REMARK = re.compile(r"remark:\s+([A-Za-z][A-Za-z /\[\]]*?):\s+(\S+) \[-Rpass-analysis=kernel-resource-usage\]")
 
 
 def sources():
@@ -35,13 +41,29 @@ def _compile(src, objdir, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(line for line in r.stdout.splitlines()
-                    if "packed-fp32-ops" not in line)   # the host pass does not know the device feature: harmless
+    kernels, name, keep, skip = {}, None, [], 0
+    for line in r.stdout.splitlines():
+        if "packed-fp32-ops" in line:                   # the host pass does not know the device feature: harmless
+            continue
+        m = _REMARK.search(line)
+        if m:
+            skip = 2                                    # the remark's two lines of source context
+            if m.group(1) == "Function Name":
+                name = m.group(2)
+                kernels[name] = {}
+            elif name is not None:
+                v = m.group(2)
+                kernels[name][m.group(1).strip()] = int(v) if v.isdigit() else v
+        elif skip:
+            skip -= 1
+        else:
+            keep.append(line)
+    out = "\n".join(keep)
     if r.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, out))
     if verbose and out.strip():
         print(out, flush=True)
-    return obj
+    return obj, kernels
 
 
 def build(verbose=True, jobs=None):
@@ -51,7 +73,10 @@ def build(verbose=True, jobs=None):
     srcs = sources()
     jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2) - 1), 8)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(lambda s: _compile(s, objdir, verbose), srcs))
+        done = list(pool.map(lambda s: _compile(s, objdir, verbose), srcs))
+    objs = [o for o, _ in done]
+    with open(RESOURCES, "w") as f:
+        json.dump({os.path.basename(s): k for s, (_, k) in zip(srcs, done)}, f, indent=1, sort_keys=True)
     cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=" + ARCH, "-o", LIBPATH] + objs
     if verbose:
         print(" ".join(cmd), flush=True)

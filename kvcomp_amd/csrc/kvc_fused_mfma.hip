@@ -447,8 +447,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     // bits the lengths of a two-symbol entry go to (header word 6: OR of all the patterns)
     const bool pairs = fast_book && a.pair_bits != 0 && pbits <= (uint32_t)a.pair_bits && pbits <= 10u &&
                        (1u << pbits) <= (uint32_t)a.table_words && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
-    // codes of 6 or 7 bits: two-byte entries (see kvc_mfma_dot), where no symbol's fp16 pattern needs its five lowest bits
-    const bool half_table = fast_book && !pairs && lbits >= 6u && a.half_table != 0 && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
+    // codes of 6 or 7 bits: two-byte entries (see kvc_mfma_dot), where no symbol's fp16 pattern needs its five lowest bits.
+    // Not for V tiles that may straddle two heads: with that loop beside the others the kernel needs one register more
+    // than six waves per SIMD leave it, and the compiler then spills in the per-tile path of every variant.
+    constexpr bool HALF_OK = KIND != 4;
+    const bool half_table = HALF_OK && fast_book && !pairs && lbits >= 6u && a.half_table != 0 && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
     const uint32_t lead_bits = half_table ? 1u : 2u;                   // bits of the window below the table index
     if (pairs) {
         // the one-symbol table goes to the (not yet used) per-wave areas; the two-symbol table is derived from it
@@ -543,7 +546,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                     if (per == 16) kvc_mfma_dot<8, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
                     else if (per == 12) kvc_mfma_dot<6, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, n_main, bptr, msptr, acc, holder);
                     const int rest = per == 8 ? n : n - n_main;
-                    if (rest && half_table) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST, true>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
+                    if (HALF_OK && rest && half_table) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST, HALF_OK>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                     else if (rest) kvc_mfma_dot<4, SK, NM, ROUNDED, BCAST>(sbase, u, fe, mask4, rest, bptr, msptr, acc, holder);
                 }
             };
