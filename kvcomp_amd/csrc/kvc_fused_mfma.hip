@@ -116,13 +116,30 @@ __device__ __forceinline__ void kvc_split_weight(float v, float &hi, float &lo)
     lo = (v - hi) * KVC_LO_SCALE;
 }
 
+// Rounded mode: the minima of a lane's two elements as two fp16, and their two scales, in the order the decode loops read
+// them.  Where both elements' parameters came in one word each (wave-uniform `pmode`), the scales are that word and the
+// two int8 minima are converted together: the byte m ^ 0x80 = m + 128 under the byte 0x64 is the fp16 number 1152 + m.
+template <class Raw>
+__device__ __forceinline__ void kvc_mfma_min_scale_words(const Raw &raw, int s, int pmode, uint32_t &mins, uint32_t &scales)
+{
+    if (pmode == KVC_PAIR_ADJACENT) {
+        const uint32_t biased = __builtin_amdgcn_perm(0x64u, raw.mnw[s][0] ^ 0x8080u, 0x04010400u);
+        const kvc_h2 off = {(_Float16)-1152.f, (_Float16)-1152.f};
+        mins = __builtin_bit_cast(uint32_t, __builtin_bit_cast(kvc_h2, biased) + off);                              // exact
+        scales = raw.scw[s][0];
+    } else {
+        mins = kvc_half_pair((float)raw.min_int(s, 0, pmode), (float)raw.min_int(s, 1, pmode));                    // exact
+        scales = raw.scale_bits(s, 0, pmode) | (raw.scale_bits(s, 1, pmode) << 16);
+    }
+}
+
 // Build the operand tables of a fetched tile; returns per query head the constant term sum_i min_i weight_i of this
 // lane's head slot (zero in rounded mode) and the power of two the weights were divided by to stay inside fp16.
 template <int REP, int KIND, bool ROUNDED>
 __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int row, int col, int lane,
                                                    const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw,
                                                    uint32_t *btab, uint32_t *mstab, float (&bias)[REP], float &unscale,
-                                                   int &sel_out)
+                                                   int &sel_out, bool &lo_used)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     constexpr int NM = kvc_mfma_sets(REP);
@@ -133,6 +150,48 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
     const bool straddles = SLOTS == 2 && (col * KVC_WAVE) % D + KVC_WAVE > D;      // wave-uniform
     const bool live = KIND != 0 || 2 * lane < D;
     const int pmode = kvc_pair_mode<KIND>(a);
+    // Rounded mode without the softmax: the weights are the caller's fp16 values (q, or p).  Unless one of them is
+    // subnormal they are their own high parts and the low parts are zero: the words go to the table as they were
+    // loaded, and the low columns stay (or are made) zero.
+    if constexpr (ROUNDED && !KvcGeom<KIND>::SOFTMAX) {
+        bool subnormal = false;
+#pragma unroll
+        for (int s = 0; s < SLOTS; s++) {
+            if (s == 1 && !straddles) continue;
+#pragma unroll
+            for (int r = 0; r < REP; r++) {
+                const kvc_h2 w = __builtin_bit_cast(kvc_h2, raw.x[s][r][0]);
+                subnormal = subnormal | __builtin_amdgcn_classh(w.x, 0x90) | __builtin_amdgcn_classh(w.y, 0x90);
+            }
+        }
+        if (!__any(live && subnormal)) {
+            const int g = lane >> 1, odd = lane & 1;
+            if (live) {
+#pragma unroll
+                for (int s = 0; s < SLOTS; s++) {
+                    uint32_t *bg = btab + s * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
+                    if (lo_used) {                             // low parts an earlier tile of this wave left, in either slot
+#pragma unroll
+                        for (int r = 0; r < REP; r++) bg[(((2 * r + 1) >> 2) * 4 + ((2 * r + 1) & 3)) * 2] = 0u;
+                    }
+                    if (s == 1 && !straddles) continue;
+#pragma unroll
+                    for (int r = 0; r < REP; r++) bg[(((2 * r) >> 2) * 4 + ((2 * r) & 3)) * 2] = raw.x[s][r][0];
+                    uint32_t *mg = mstab + s * T::MSTAB_SLOT_WORDS + g * 4 + odd;
+                    kvc_mfma_min_scale_words(raw, s, pmode, mg[0], mg[2]);
+                }
+            }
+            lo_used = false;
+            unscale = 1.f;
+            int sel = 0;
+            if (SLOTS == 2) sel = ((col * KVC_WAVE) % D + lane) >= D;
+            sel_out = sel;
+#pragma unroll
+            for (int r = 0; r < REP; r++) bias[r] = 0.f;
+            return;
+        }
+    }
+    lo_used = true;
     float vmax = 0.f;
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {
@@ -208,8 +267,7 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
             }
             if (ROUNDED) {
                 uint32_t *mg = mstab + s * T::MSTAB_SLOT_WORDS + g * 4 + odd;
-                mg[0] = kvc_half_pair((float)raw.min_int(s, 0, pmode), (float)raw.min_int(s, 1, pmode));           // exact
-                mg[2] = raw.scale_bits(s, 0, pmode) | (raw.scale_bits(s, 1, pmode) << 16);
+                kvc_mfma_min_scale_words(raw, s, pmode, mg[0], mg[2]);
             }
         }
     }
@@ -450,7 +508,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     // codes of 6 or 7 bits: two-byte entries (see kvc_mfma_dot), where no symbol's fp16 pattern needs its five lowest bits.
     // Not for V tiles that may straddle two heads: with that loop beside the others the kernel needs one register more
     // than six waves per SIMD leave it, and the compiler then spills in the per-tile path of every variant.
-    constexpr bool HALF_OK = KIND != 4;
+    constexpr bool HALF_OK = SLOTS == 1;
     const bool half_table = HALF_OK && fast_book && !pairs && lbits >= 6u && a.half_table != 0 && (lut_g[6] & KVC_PAIR_LEN_MASK) == 0u;
     const uint32_t lead_bits = half_table ? 1u : 2u;                   // bits of the window below the table index
     if (pairs) {
@@ -491,10 +549,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
     kvc_fetch_tile<REP, KIND>(a, row, col, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
     float bias[REP], unscale;
     int sel = 0;
+    bool lo_used = false;          // wave-uniform: the low-part columns of the operand table hold something (they start as zeros)
     uint32_t first, longest;
     KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
     if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;       // one or two bits before the lane's first code
-    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col, lane, raw, btab, mstab, bias, unscale, sel);
+    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col, lane, raw, btab, mstab, bias, unscale, sel, lo_used);
     kvc_wave_sync();
     for (int it = 0; it < ntiles; it++) {
         // the arguments are read again per tile rather than kept in scalar registers through the decode loops (the
@@ -564,8 +623,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
                 for (int rr = 0; rr < REP; rr++)
                     if (rr == r) bs = bias[rr];
 #pragma unroll
-                for (int i = 0; i < 4; i++)
-                    res[i] = fmaf(kvc_quad_next(acc[s][i]), 1.f / KVC_LO_SCALE, acc[s][i]);
+                for (int i = 0; i < 4; i++) res[i] = acc[s][i];
+                if (lo_used) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) res[i] = fmaf(kvc_quad_next(acc[s][i]), 1.f / KVC_LO_SCALE, acc[s][i]);
+                }
                 if (!ROUNDED) {                        // rounded mode folds nothing into a constant and never rescales
 #pragma unroll
                     for (int i = 0; i < 4; i++) res[i] = res[i] * unscale + bs;
@@ -602,7 +664,7 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             asm volatile("" : "+v"(lane_s));
             st = kvc_stage_payload(a, lane_s, raw, pack, first, longest);
             if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;
-            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row_next, col_next, lane_s, raw, btab, mstab, bias, unscale, sel);
+            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row_next, col_next, lane_s, raw, btab, mstab, bias, unscale, sel, lo_used);
             kvc_wave_sync();
         }
         row = row_next;

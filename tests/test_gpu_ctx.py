@@ -94,6 +94,47 @@ def test_fused_mat_vec_mul_against_dense(is_k, mode):
     assert ms > 0
 
 
+@pytest.mark.parametrize("D", [128, 96])
+def test_fused_matvecs_with_subnormal_weights_in_some_heads(D):
+    """In the default arithmetic the matrix-core kernels hand fp16 weights (q, or p without the softmax) to the matrix
+    cores as the words they were loaded as, unless a weight of the tile is subnormal: then the tile's weights are split
+    into a high part (zero where subnormal) and a low part scaled into the normal range.  Heads alternate here between
+    ordinary and entirely subnormal weights, so a wave that works through several tiles switches between the two
+    forms: every head's result must match the dense product (a head whose low parts were lost would come out zero),
+    and runs of three tiles must give the bits of single tiles."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd import attention as A
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant")
+    T, B, H = 640, 2, 6
+    kctx, vctx = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+    kctx.store(S.synth_k(T, B, H, D).to(DEV))
+    vctx.store(S.synth_v(T, B, H, D).to(DEV))
+    assert 1 <= kctx.max_code_bits <= 7 and 1 <= vctx.max_code_bits <= 7      # the matrix-core kernels' range
+    q, p = S.synth_q(B, H, D).to(DEV), S.synth_p(B, H, T).to(DEV).clamp_min(2e-4)      # (no subnormal p in the even heads)
+    for w in (q, p):                                       # odd heads: a few 1e-5, below fp16's smallest normal 6.1e-5
+        small = w[:, 1::2].float()
+        w[:, 1::2] = (small / small.abs().max() * 5e-5).to(torch.float16)
+        assert (w[:, 1::2].float().abs() < 6.1e-5).all() and (w[:, 1::2] != 0).any()
+    for ctx, w, fn in ((kctx, q, A.k_scores), (vctx, p, A.v_partials)):
+        lut = A.build_lut(ctx.decode_codebook, ctx.tree_format)
+        out = {}
+        for tpw in (1, 3):
+            was = _lib.set_option("fused_tiles_per_wave", tpw)
+            try:
+                out[tpw] = fn(ctx, lut, w)[0]
+            finally:
+                _lib.set_option("fused_tiles_per_wave", was)
+        assert torch.equal(out[1], out[3])
+        dense = ctx.get_only_compressed()[0].float()
+        if ctx.is_k:
+            got, ref = out[1], torch.einsum("tbhd,bhd->bht", dense, w.float())
+        else:
+            got, ref = out[1].sum(dim=0), torch.einsum("tbhd,bht->bhd", dense, w.float())
+        err, scale = (got - ref).abs().amax(dim=2), ref.abs().amax(dim=2)
+        assert (scale > 0).all() and (err <= 1e-3 * scale).all(), (err / scale).max()
+
+
 def test_prefill_then_append_one_token_at_a_time():
     from kvcomp_amd.ctx import KVCompCtx
     _config(v_recent=256)
