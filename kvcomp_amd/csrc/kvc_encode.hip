@@ -863,16 +863,26 @@ struct KvcOncePending {
     KvcFirstLooks looks;
 };
 
-// Look back for a tile whose size has been published, publish its block_info and write its payload from the LDS
-// image (which starts on a word; the payload lands p.head bytes into an aligned word).  Returns error bits.
+// Find where a tile whose size has been published goes (by looking back, or -- `follows` -- right behind the tile
+// before it, which this wave has just placed at follows_off), publish its block_info and write its payload from the LDS
+// image (which starts on a word; the payload lands p.head bytes into an aligned word).  Returns error bits; *off_out
+// receives the tile's global offset.
 __device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const KvcOncePending &pd, const uint32_t *image, uint32_t base,
-                                                   int lane, int *polls)
+                                                   int lane, int *polls, uint32_t *off_out, bool follows = false, uint32_t follows_off = 0)
 {
     const int64_t tile = pd.tile;
     const uint32_t bn = pd.bn;
-    uint32_t in_group = pd.in_group;
-    if (!pd.in_group_known) in_group = kvc_look_back_in_group(a, tile, bn, lane, pd.looks.tile_word, polls);
-    const uint32_t off = base + in_group + kvc_look_back_groups(a, tile, in_group + bn, lane, pd.looks.group_word, polls);
+    uint32_t off;
+    if (follows) {
+        off = follows_off;
+        if (((tile & 63) == 63 || tile == a.tiles - 1) && lane == 0)      // this wave speaks for its group: the group's end
+            kvc_status_store(kvc_group_words(a) + (tile >> 6), kvc_group_word(off + bn - base, 0u));
+    } else {
+        uint32_t in_group = pd.in_group;
+        if (!pd.in_group_known) in_group = kvc_look_back_in_group(a, tile, bn, lane, pd.looks.tile_word, polls);
+        off = base + in_group + kvc_look_back_groups(a, tile, in_group + bn, lane, pd.looks.group_word, polls);
+    }
+    *off_out = off;
     uint32_t err = 0;
     const bool gave_up = *polls > KVC_LOOKBACK_POLLS;
     if (lane == 0) kvc_status_store(reinterpret_cast<uint64_t *>(a.block_infos) + tile, kvc_bi_word(off, bn, 0u));
@@ -896,13 +906,14 @@ __device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const
 }
 
 // FRONT 0: uint8 symbols in; 1: fp16 K tile (quantized here); 2: fp16 V tile.
-// A wave works through `run` (one or two) consecutive tiles.  For each it counts (symbols -> codes and lengths, thread_infos),
-// publishes the size and asks for the words its look-back will read; then it places the tile before this one (look
-// back, block_info, payload out of the wave's second LDS area to its byte position) and packs this tile's payload
-// into that area, as an image that starts on a word (where the payload goes is not needed for that).  So a tile is
-// placed one tile's count after its size was published, when the tiles before it have published theirs: with the
-// look-back right behind the count, a tile waits 10 us on average for the slowest of the thousands of tiles in flight
-// before it (measured), as long as the rest of its work takes.
+// A wave works through `run` (one or two) consecutive tiles.  For each it counts (symbols -> codes and lengths,
+// thread_infos), publishes the size, asks for the words its look-back will read and packs the payload into LDS as an
+// image that starts on a word (where the payload goes is not needed for that).  The first tile of a run of two stays in
+// the wave's second LDS area until the second is packed too; then one look-back finds the first tile's place, the second
+// follows right behind it, and both are written out.  So a tile is placed a whole tile's work after its size was
+// published, when the tiles before it have published theirs: with the look-back right behind the count, a tile waits
+// 10 us on average for the slowest of the thousands of tiles in flight before it (measured), as long as the rest of
+// its work takes.
 // Dynamic LDS: the encode table (one for the workgroup, or one per wave when tile rows have codebooks of their own:
 // then run = 1), then per wave the tile of symbols, for V the tokens' constants, and the kept payload image.
 template <int FRONT>
@@ -984,19 +995,14 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
         KvcOncePending cur;
         cur.tile = tile;
         cur.bn = bn;
-        cur.looks = kvc_look_back_ask(a.e, tile, lane);
         // the wave that speaks for a group must not sit on the group's size (the groups after it wait for that word,
         // and so would, one after the other, the waves that speak for them): it adds up its group at once
         cur.in_group_known = (tile & 63) == 63 || tile == a.e.tiles - 1;
         cur.in_group = 0;
+        cur.looks.tile_word = cur.looks.group_word = 0ull;
+        if (pd.tile < 0 || cur.in_group_known) cur.looks = kvc_look_back_ask(a.e, tile, lane);    // (a tile that follows a kept one looks at nothing)
         if (cur.in_group_known) cur.in_group = kvc_look_back_in_group(a.e, tile, bn, lane, cur.looks.tile_word, &polls);
         cur.packs = bn <= (uint32_t)KVC_MAX_TILE_BYTES;
-        // the tile before this one: its words have had this tile's count to arrive
-        if (pd.tile >= 0) {
-            err |= kvc_once_place(a.e, pd, kept, base, lane, &polls);
-            kvc_wave_lds_sync();                           // the kept image is read
-        }
-        pd.tile = -1;
         const bool keep = bn <= (uint32_t)KEEP_BYTES && it + 1 < run && tile + 1 < a.e.tiles;
         uint32_t *image = keep ? kept : reinterpret_cast<uint32_t *>(s_sym);
         if (cur.packs) {
@@ -1029,11 +1035,18 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
             kvc_wave_lds_sync();
         }
         if (keep) {
-            pd = cur;                                      // placed after the next tile is counted
-        } else {
-            err |= kvc_once_place(a.e, cur, image, base, lane, &polls);      // the wave's last tile, or too large to keep
-            kvc_wave_lds_sync();                           // the image is read: the area may take the next tile
+            pd = cur;                                      // placed together with the next tile
+            continue;
         }
+        uint32_t off = 0;
+        if (pd.tile >= 0) {                                // the kept tile, whose words have had this tile's work to arrive
+            err |= kvc_once_place(a.e, pd, kept, base, lane, &polls, &off);
+            err |= kvc_once_place(a.e, cur, image, base, lane, &polls, &off, true, off + pd.bn);
+            pd.tile = -1;
+        } else {                                           // a run of one, or the tile before was too large to keep
+            err |= kvc_once_place(a.e, cur, image, base, lane, &polls, &off);
+        }
+        kvc_wave_lds_sync();                               // the images are read: the areas may take the next tiles
     }
     if (lane == 0 && tile0 < a.e.tiles) {
         if (err) atomicOr(&s_err, err);
