@@ -707,6 +707,17 @@ constexpr int KVC_ONCE_BASE_WORD = 32;               // copy of status[KVC_ENC_S
 constexpr int KVC_ONCE_PART_WORD = 64, KVC_ONCE_PART_LINES = 32, KVC_ONCE_PART_STRIDE = 32;   // {error bits, largest tile, longest stream}
 constexpr int KVC_ONCE_GROUP_WORD = KVC_ONCE_PART_WORD + KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE;
 constexpr int KVC_ONCE_MAX_GROUPS = (int)((KVC_WS_SLOT_BYTES - KVC_ONCE_GROUP_WORD * 4) / 8);
+// Tiles per group: seven workgroups of a run-of-two launch, not eight.  Workgroups go to the chip's eight dies in turn,
+// and the wave of a group's last tile waits for its whole group before it publishes the group's size: with groups of
+// eight workgroups all of those waves sit on one die, that die falls behind, and the seven others wait for it at every
+// group (measured: 10 us per wave there, 3 us on the die with the last tiles).
+constexpr int KVC_ONCE_GROUP_TILES = 56;
+static_assert(KVC_ONCE_GROUP_TILES <= KVC_WAVE && KVC_ONCE_GROUP_TILES % 2 == 0, "one look of 64 lanes covers a group; a run of two stays inside one");
+__device__ __forceinline__ int64_t kvc_once_group(int64_t tile) { return (int64_t)((uint32_t)tile / (uint32_t)KVC_ONCE_GROUP_TILES); }
+__device__ __forceinline__ bool kvc_once_closes(const KvcEncodeArgs &a, int64_t tile)
+{
+    return (uint32_t)tile % (uint32_t)KVC_ONCE_GROUP_TILES == (uint32_t)KVC_ONCE_GROUP_TILES - 1u || tile == a.tiles - 1;
+}
 
 __device__ __forceinline__ uint64_t kvc_bi_word(uint32_t offset, uint32_t byte_num, uint32_t state)
 {
@@ -731,7 +742,7 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_mark_kernel(KvcEncodeArgs a
 {
     const int64_t tile = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
     if (tile < a.tiles) reinterpret_cast<uint64_t *>(a.block_infos)[tile] = kvc_bi_word(0u, 0u, KVC_BI_NOT_READY);
-    if (tile < (a.tiles + KVC_WAVE - 1) / KVC_WAVE) kvc_group_words(a)[tile] = kvc_group_word(0u, KVC_BI_NOT_READY);
+    if (tile < (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES) kvc_group_words(a)[tile] = kvc_group_word(0u, KVC_BI_NOT_READY);
     if (blockIdx.x == 0) {
         for (int i = threadIdx.x; i < KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE; i += KVC_WG) a.status[KVC_ONCE_PART_WORD + i] = 0u;
         if (threadIdx.x == 0) a.status[KVC_ONCE_BASE_WORD] = a.status[KVC_ENC_ST_BASE];
@@ -773,10 +784,10 @@ struct KvcFirstLooks {
 __device__ __forceinline__ KvcFirstLooks kvc_look_back_ask(const KvcEncodeArgs &a, int64_t tile, int lane)
 {
     const uint64_t *bi64 = reinterpret_cast<const uint64_t *>(a.block_infos);
-    const int64_t group = tile >> 6;
-    const int r = (int)(tile & 63);
+    const int64_t group = kvc_once_group(tile);
+    const int r = (int)(tile - group * KVC_ONCE_GROUP_TILES);
     KvcFirstLooks f;
-    f.tile_word = lane < r ? kvc_status_load(bi64 + (group << 6) + lane) : 0ull;
+    f.tile_word = lane < r ? kvc_status_load(bi64 + group * KVC_ONCE_GROUP_TILES + lane) : 0ull;
     f.group_word = group - 1 - lane >= 0 ? kvc_status_load(kvc_group_words(a) + group - 1 - lane) : kvc_group_word(0u, 0u);
     return f;
 }
@@ -787,8 +798,8 @@ __device__ __forceinline__ uint32_t kvc_look_back_in_group(const KvcEncodeArgs &
                                                            int *polls)
 {
     const uint64_t *bi64 = reinterpret_cast<const uint64_t *>(a.block_infos);
-    const int64_t group = tile >> 6;
-    const int r = (int)(tile & 63);
+    const int64_t group = kvc_once_group(tile);
+    const int r = (int)(tile - group * KVC_ONCE_GROUP_TILES);
     uint32_t in_group = 0;
     uint64_t w = first_look;
     while (r > 0) {
@@ -798,9 +809,9 @@ __device__ __forceinline__ uint32_t kvc_look_back_in_group(const KvcEncodeArgs &
         }
         if (++*polls > KVC_LOOKBACK_POLLS) break;
         __builtin_amdgcn_s_sleep(2);
-        w = lane < r ? kvc_status_load(bi64 + (group << 6) + lane) : 0ull;
+        w = lane < r ? kvc_status_load(bi64 + group * KVC_ONCE_GROUP_TILES + lane) : 0ull;
     }
-    if ((r == 63 || tile == a.tiles - 1) && lane == 0)     // this wave speaks for its group
+    if (kvc_once_closes(a, tile) && lane == 0)             // this wave speaks for its group
         kvc_status_store(kvc_group_words(a) + group, kvc_group_word(in_group + bn, KVC_BI_SIZE));
     return in_group;
 }
@@ -811,7 +822,7 @@ __device__ __forceinline__ uint32_t kvc_look_back_groups(const KvcEncodeArgs &a,
                                                          uint64_t first_look, int *polls)
 {
     uint64_t *groups = kvc_group_words(a);
-    const int64_t group = tile >> 6;
+    const int64_t group = kvc_once_group(tile);
     uint32_t before = 0;
     int64_t j = group - 1;                                 // nearest group not yet accounted for
     uint64_t w = first_look;                               // taken at j = group - 1
@@ -830,7 +841,7 @@ __device__ __forceinline__ uint32_t kvc_look_back_groups(const KvcEncodeArgs &a,
         const int64_t idx = j - lane;
         w = idx >= 0 ? kvc_status_load(groups + idx) : kvc_group_word(0u, 0u);   // in front of the first group: nothing, and known
     }
-    if (((tile & 63) == 63 || tile == a.tiles - 1) && lane == 0)
+    if (kvc_once_closes(a, tile) && lane == 0)
         kvc_status_store(groups + group, kvc_group_word(before + in_group_and_own, 0u));
     return before;
 }
@@ -875,8 +886,8 @@ __device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const
     uint32_t off;
     if (follows) {
         off = follows_off;
-        if (((tile & 63) == 63 || tile == a.tiles - 1) && lane == 0)      // this wave speaks for its group: the group's end
-            kvc_status_store(kvc_group_words(a) + (tile >> 6), kvc_group_word(off + bn - base, 0u));
+        if (kvc_once_closes(a, tile) && lane == 0)         // this wave speaks for its group: the group's end
+            kvc_status_store(kvc_group_words(a) + kvc_once_group(tile), kvc_group_word(off + bn - base, 0u));
     } else {
         uint32_t in_group = pd.in_group;
         if (!pd.in_group_known) in_group = kvc_look_back_in_group(a, tile, bn, lane, pd.looks.tile_word, polls);
@@ -997,7 +1008,7 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
         cur.bn = bn;
         // the wave that speaks for a group must not sit on the group's size (the groups after it wait for that word,
         // and so would, one after the other, the waves that speak for them): it adds up its group at once
-        cur.in_group_known = (tile & 63) == 63 || tile == a.e.tiles - 1;
+        cur.in_group_known = kvc_once_closes(a.e, tile);
         cur.in_group = 0;
         cur.looks.tile_word = cur.looks.group_word = 0ull;
         if (pd.tile < 0 || cur.in_group_known) cur.looks = kvc_look_back_ask(a.e, tile, lane);    // (a tile that follows a kept one looks at nothing)
@@ -1166,7 +1177,7 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     // and the one-pass kernel runs at three waves per SIMD; the option's values 2 and 3 still send them through one pass)
     const int one_pass = kvc_option(KVC_OPT_ENCODE_ONE_PASS);
     if ((src ? one_pass != 0 : one_pass > 1) && ((uintptr_t)c.d_block_infos & 7) == 0 &&
-        (a.tiles + KVC_WAVE - 1) / KVC_WAVE <= KVC_ONCE_MAX_GROUPS) {
+        (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES <= KVC_ONCE_MAX_GROUPS) {
         if (!src) sa.e = a;
         const int front = !src ? 0 : is_k ? 1 : 2;
         const size_t lds = (size_t)(a.rows_per_codebook ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2) +
