@@ -514,19 +514,26 @@ __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile,
     for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
 }
 
-// The count pass's variant: the lane keeps its two channels of all 64 tokens in registers (64 loads in flight, one walk
-// over the tile), finds the groups' minima and maxima there (packed fp16 min / max), publishes the group parameters
-// and quantizes.
-__device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t (&v)[32])
+// The count pass's variant: the lane keeps its two channels of all 64 tokens in registers (kvc_front_k_load: 64 loads in
+// flight, one walk over the tile), finds the groups' minima and maxima there (packed fp16 min / max), publishes the group
+// parameters and quantizes.
+__device__ __forceinline__ void kvc_front_k_load(const KvcStoreArgs &a, int64_t tile, int lane, uint32_t (&raw)[KVC_WAVE])
+{
+    const int64_t stride = a.e.stride;
+    const int D = a.D;
+    const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
+    const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (2 * lane < D ? 2 * lane : 0);
+#pragma unroll
+    for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + t * stride);
+}
+
+__device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, const uint32_t (&raw)[KVC_WAVE],
+                                                 uint32_t (&v)[32])
 {
     const int64_t stride = a.e.stride;
     const int D = a.D, RS = D + 4;
     const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
     const bool act = 2 * lane < D;
-    const __half *p = a.x + (row * KVC_WAVE) * stride + col * D + (act ? 2 * lane : 0);
-    uint32_t raw[KVC_WAVE];
-#pragma unroll
-    for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + t * stride);
     KvcGroupParams g0, g1;
     if (a.mask == KVC_MASK_CHANNEL) {
         const int64_t g = row * stride + col * D + (act ? 2 * lane : 0);
@@ -634,8 +641,13 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
     __syncthreads();
     if (tile < a.e.tiles) {
         uint32_t v[32];
-        if (IS_K) kvc_front_k_once(a, tile, lane, s_sym[wave], v);
-        else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+        if (IS_K) {
+            uint32_t raw[KVC_WAVE];
+            kvc_front_k_load(a, tile, lane, raw);
+            kvc_front_k_once(a, tile, lane, s_sym[wave], raw, v);
+        } else {
+            kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+        }
         const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len[wave], &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
     }
@@ -956,14 +968,22 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
     int polls = 0;
     KvcOncePending pd;
     pd.tile = -1;
+    uint32_t raw[KVC_WAVE];                                // FRONT 1: a K tile as loaded, two channels of 64 tokens per lane
 #pragma unroll 1
     for (int it = 0; it < run; it++) {
         const int64_t tile = tile0 + it;
         if (tile >= a.e.tiles) break;
         uint32_t v[32];
-        if (FRONT == 1) kvc_front_k_once(a, tile, lane, s_sym, v);
-        else if (FRONT == 2) kvc_front_v(a, tile, lane, s_sym, s_par, v);
-        else kvc_load_vector(a.e, tile, lane, v);
+        if constexpr (FRONT == 1) {
+            // the loads of the run's second tile are on their way while the first is counted and packed
+            if (it == 0) kvc_front_k_load(a, tile, lane, raw);
+            kvc_front_k_once(a, tile, lane, s_sym, raw, v);
+            if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_k_load(a, tile + 1, lane, raw);
+        } else if constexpr (FRONT == 2) {
+            kvc_front_v(a, tile, lane, s_sym, s_par, v);
+        } else {
+            kvc_load_vector(a.e, tile, lane, v);
+        }
         kvc_wave_lds_sync();                               // every lane holds its vector: the tile area is free
         uint32_t bits = 0;
         uint32_t gl[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u}; // short codes: the four group lengths of registers 4 i .. 4 i + 3
