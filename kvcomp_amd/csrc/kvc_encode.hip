@@ -583,14 +583,24 @@ __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t 
 // then reads channel c's vector.  Group parameters are per token (KVC_MASK_V_TOKEN) or per (token, batch
 // entry) (KVC_MASK_SIM_TOKEN; the tile lies inside one batch entry); the wave first stages its 128 triples
 // {scale, 1 / scale, min} in LDS.
-__device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t *s_par,
-                                            uint32_t (&v)[32])
+__device__ __forceinline__ void kvc_front_v_load(const KvcStoreArgs &a, int64_t tile, int lane, uint32_t (&raw)[KVC_WAVE])
 {
     const int64_t stride = a.e.stride;
+    const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
+    const int pr = lane & 31, half = lane >> 5;
+    const __half *p = a.x + (row * KVC_V_TOKENS + 64 * half) * stride + col * KVC_WAVE + 2 * pr;
+#pragma unroll
+    for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + (int64_t)t * stride);
+}
+
+// raw: the lane's channel pair of its 64 tokens, as kvc_front_v_load fetched them (all 64 loads in flight at once: taken
+// four at a time between the quantizing, the loop waited for memory sixteen times)
+__device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t *s_par,
+                                            const uint32_t (&raw)[KVC_WAVE], uint32_t (&v)[32])
+{
     constexpr int RS = KVC_V_TOKENS + 4;
     const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
     const int pr = lane & 31, half = lane >> 5;
-    const int64_t ch = col * KVC_WAVE + 2 * pr;
     const int64_t b = (col * KVC_WAVE) / ((int64_t)a.H * a.D);
 #pragma unroll
     for (int k = 0; k < 2; k++) {
@@ -603,8 +613,7 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const __half *p = a.x + (row * KVC_V_TOKENS + 64 * half) * stride + ch;
-#pragma unroll 2
+#pragma unroll
     for (int jj = 0; jj < 16; jj++) {
         uint32_t u[4];
 #pragma unroll
@@ -612,7 +621,7 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
             const int t = 64 * half + 4 * jj + k;
             const uint4 c = *reinterpret_cast<const uint4 *>(s_par + 4 * t);
             const KvcPackedParams pp = {c.x, c.y, c.z, c.w};
-            u[k] = kvc_quant_pair_biased(*reinterpret_cast<const uint32_t *>(p + (int64_t)(4 * jj + k) * stride), pp);
+            u[k] = kvc_quant_pair_biased(raw[4 * jj + k], pp);
         }
         // a01 = {channel 2 pr, 2 pr + 1 of token 4 jj | the same of token 4 jj + 1}; then four tokens of each channel
         const uint32_t a01 = kvc_low_bytes4(u[0], u[1]), a23 = kvc_low_bytes4(u[2], u[3]);
@@ -646,7 +655,9 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_count_kernel(KvcStoreArgs a)
             kvc_front_k_load(a, tile, lane, raw);
             kvc_front_k_once(a, tile, lane, s_sym[wave], raw, v);
         } else {
-            kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+            uint32_t raw[KVC_WAVE];
+            kvc_front_v_load(a, tile, lane, raw);
+            kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], raw, v);
         }
         const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len[wave], &s_err);
         if (lane == 0) atomicMax(&s_longest, longest);
@@ -673,8 +684,13 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
     if (!p.ok) return;                                 // wave-uniform; nothing below involves another wave
     uint32_t *image = reinterpret_cast<uint32_t *>(s_sym[wave]);
     uint32_t v[32];
-    if (IS_K) kvc_front_k(a, tile, lane, s_sym[wave], v);
-    else kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], v);
+    if (IS_K) {
+        kvc_front_k(a, tile, lane, s_sym[wave], v);
+    } else {
+        uint32_t raw[KVC_WAVE];
+        kvc_front_v_load(a, tile, lane, raw);
+        kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], raw, v);
+    }
     kvc_wave_lds_sync();                               // every lane holds its vector: the tile can be overwritten
     const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
     for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
@@ -968,7 +984,7 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
     int polls = 0;
     KvcOncePending pd;
     pd.tile = -1;
-    uint32_t raw[KVC_WAVE];                                // FRONT 1: a K tile as loaded, two channels of 64 tokens per lane
+    uint32_t raw[KVC_WAVE];                                // a tile as loaded from fp16: two channels of 64 tokens per lane
 #pragma unroll 1
     for (int it = 0; it < run; it++) {
         const int64_t tile = tile0 + it;
@@ -980,7 +996,9 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
             kvc_front_k_once(a, tile, lane, s_sym, raw, v);
             if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_k_load(a, tile + 1, lane, raw);
         } else if constexpr (FRONT == 2) {
-            kvc_front_v(a, tile, lane, s_sym, s_par, v);
+            if (it == 0) kvc_front_v_load(a, tile, lane, raw);
+            kvc_front_v(a, tile, lane, s_sym, s_par, raw, v);
+            if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_v_load(a, tile + 1, lane, raw);
         } else {
             kvc_load_vector(a.e, tile, lane, v);
         }
