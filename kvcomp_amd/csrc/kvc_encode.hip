@@ -1210,11 +1210,13 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
         sa.scale_f16 = reinterpret_cast<__half *>(src->scale_f16);
     }
     hipLaunchKernelGGL(kvc_encode_init_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
-    // one pass (each wave counts, places and emits its tile) where the block_infos can serve as 64-bit status words
-    // (from uint8 symbols the two passes are the faster way, 1.1 - 1.5 times on MI355X: there is no quantizing to save,
-    // and the one-pass kernel runs at three waves per SIMD; the option's values 2 and 3 still send them through one pass)
+    // one pass (each wave counts, places and emits its tile) where the block_infos can serve as 64-bit status words.
+    // From uint8 symbols there is no quantizing to save and the one-pass kernel runs at three waves per SIMD: measured on
+    // MI355X at 65 536 tiles, K symbols encode 1.17 times faster in one pass and V symbols 1.4 times faster in two, so
+    // by default only large K calls take the one pass (the option's values 2 and 3 send every call through it).
     const int one_pass = kvc_option(KVC_OPT_ENCODE_ONE_PASS);
-    if ((src ? one_pass != 0 : one_pass > 1) && ((uintptr_t)c.d_block_infos & 7) == 0 &&
+    const bool symbols_in_one_pass = one_pass > 1 || (one_pass == 1 && is_k && a.tiles >= 8192);
+    if ((src ? one_pass != 0 : symbols_in_one_pass) && ((uintptr_t)c.d_block_infos & 7) == 0 &&
         (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES <= KVC_ONCE_MAX_GROUPS) {
         if (!src) sa.e = a;
         const int front = !src ? 0 : is_k ? 1 : 2;
