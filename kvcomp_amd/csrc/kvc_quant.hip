@@ -181,6 +181,44 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel8_kernel(KvcQuantArgs
         kvc_quant_store8<1>(a, base + t * stride, *reinterpret_cast<const uint4 *>(p + t * stride), gp);
 }
 
+// Per-channel groups over blocks of 64 tokens, symbols (and parameters) out: a thread keeps its two channels of all
+// 64 tokens in registers, so the block is read once (64 loads in flight), finds minima and maxima with packed fp16
+// min / max and quantizes two channels per instruction (kvc_quant_pair_biased: the same symbols as the fp32 chain for
+// every fp16 input, see kvc_quant_math.h).
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_once_kernel(KvcQuantArgs a)
+{
+    const int64_t stride = a.B * a.H * a.D;
+    const int64_t pairs = stride >> 1;
+    const int64_t gid = (int64_t)blockIdx.x * KVC_WG + threadIdx.x;
+    if (gid >= a.NB * pairs) return;
+    const int64_t nb = gid / pairs, c = (gid - nb * pairs) * 2;
+    const int64_t base = nb * KVC_WAVE * stride + c;
+    const __half *p = a.x + base;
+    uint32_t raw[KVC_WAVE];
+#pragma unroll
+    for (int t = 0; t < KVC_WAVE; t++) raw[t] = *reinterpret_cast<const uint32_t *>(p + t * stride);
+    kvc_half2 mn = __builtin_bit_cast(kvc_half2, raw[0]), mx = mn;
+#pragma unroll
+    for (int t = 1; t < KVC_WAVE; t++) {
+        const kvc_half2 x = __builtin_bit_cast(kvc_half2, raw[t]);
+        mn = __builtin_elementwise_min(mn, x);
+        mx = __builtin_elementwise_max(mx, x);
+    }
+    const uint32_t mnw = __builtin_bit_cast(uint32_t, mn), mxw = __builtin_bit_cast(uint32_t, mx);
+    const KvcGroupParams g0 = kvc_group_params(kvc_half_lo(mnw), kvc_half_lo(mxw), a.eb);
+    const KvcGroupParams g1 = kvc_group_params(kvc_half_hi(mnw), kvc_half_hi(mxw), a.eb);
+    const int64_t g = nb * stride + c;
+    kvc_quant_publish(a, g, g0);
+    kvc_quant_publish(a, g + 1, g1);
+    const KvcPackedParams pp = kvc_packed_params(g0, g1);
+    uint8_t *out = a.sym + base;
+#pragma unroll
+    for (int t = 0; t < KVC_WAVE; t++) {
+        const uint32_t u = kvc_quant_pair_biased(raw[t], pp);
+        *reinterpret_cast<uint16_t *>(out + t * stride) = (uint16_t)kvc_low_bytes4(u, u);
+    }
+}
+
 // ---- row groups (masks 0xE, 0xC, 0x8): a group is one contiguous run of R elements; one wave per
 // group, min/max by wavefront reduction. -------------------------------------------------------------
 __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, int64_t R, int64_t groups, int wide)
@@ -211,6 +249,63 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, i
         for (int64_t i = 2 * lane; i < R; i += 2 * KVC_WAVE) {
             const __half2 v = *reinterpret_cast<const __half2 *>(p + i);
             kvc_quant_store2(a, g * R + i, __low2float(v), __high2float(v), gp, gp);
+        }
+    }
+}
+
+// Row groups of 512 to 512 NIT elements (a multiple of 8, 16-byte aligned buffers), symbols (and parameters) out: the
+// wave keeps the row in registers (NIT 16-byte loads per lane in flight), so it is read once, and quantizes two
+// elements per instruction (kvc_quant_pair_biased, as the per-channel kernel above).
+template <int NIT>
+__global__ void __launch_bounds__(KVC_WG) kvc_quant_row_once_kernel(KvcQuantArgs a, int64_t R, int64_t groups)
+{
+    const int lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * KVC_WAVES_PER_WG + (threadIdx.x >> 6);
+    if (g >= groups) return;
+    const __half *p = a.x + g * R;
+    uint4 raw[NIT];
+#pragma unroll
+    for (int j = 0; j < NIT; j++) {
+        const int64_t i = 8 * lane + 512 * j;
+        if (i < R) raw[j] = *reinterpret_cast<const uint4 *>(p + i);
+    }
+    // R >= 512 (the launcher's condition): every lane holds the row's first chunk
+    kvc_half2 mn = __builtin_bit_cast(kvc_half2, raw[0].x), mx = mn;
+    {
+        const uint32_t w[3] = {raw[0].y, raw[0].z, raw[0].w};
+#pragma unroll
+        for (int k = 0; k < 3; k++) {
+            const kvc_half2 x = __builtin_bit_cast(kvc_half2, w[k]);
+            mn = __builtin_elementwise_min(mn, x);
+            mx = __builtin_elementwise_max(mx, x);
+        }
+    }
+#pragma unroll
+    for (int j = 1; j < NIT; j++) {
+        if (8 * lane + 512 * j < R) {
+            const uint32_t w[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const kvc_half2 x = __builtin_bit_cast(kvc_half2, w[k]);
+                mn = __builtin_elementwise_min(mn, x);
+                mx = __builtin_elementwise_max(mx, x);
+            }
+        }
+    }
+    const uint32_t mnw = __builtin_bit_cast(uint32_t, mn), mxw = __builtin_bit_cast(uint32_t, mx);
+    const float lo = kvc_wave_min(fminf(kvc_half_lo(mnw), kvc_half_hi(mnw)));
+    const float hi = kvc_wave_max(fmaxf(kvc_half_lo(mxw), kvc_half_hi(mxw)));
+    const KvcGroupParams gp = kvc_group_params(lo, hi, a.eb);
+    if (lane == 0) kvc_quant_publish(a, g, gp);
+    const KvcPackedParams pp = kvc_packed_params(gp, gp);
+    uint8_t *out = a.sym + g * R;
+#pragma unroll
+    for (int j = 0; j < NIT; j++) {
+        const int64_t i = 8 * lane + 512 * j;
+        if (i < R) {
+            const uint32_t u0 = kvc_quant_pair_biased(raw[j].x, pp), u1 = kvc_quant_pair_biased(raw[j].y, pp);
+            const uint32_t u2 = kvc_quant_pair_biased(raw[j].z, pp), u3 = kvc_quant_pair_biased(raw[j].w, pp);
+            *reinterpret_cast<uint2 *>(out + i) = make_uint2(kvc_low_bytes4(u0, u1), kvc_low_bytes4(u2, u3));
         }
     }
 }
@@ -302,16 +397,23 @@ static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t
     const int64_t stride = B * H * D;
     if (quant_mask == KVC_MASK_CHANNEL) {
         const bool wide = stride % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
-        const int64_t threads = NB * (wide ? stride / 8 : stride / 2);
+        const bool once = BS == KVC_WAVE && a.sym != nullptr && a.xhat == nullptr;     // the block fits a thread's registers
+        const int64_t threads = NB * (once || !wide ? stride / 2 : stride / 8);
         const dim3 grid((unsigned)((threads + KVC_WG - 1) / KVC_WG));
-        if (wide) hipLaunchKernelGGL(kvc_quant_channel8_kernel, grid, dim3(KVC_WG), 0, stream, a);
+        if (once) hipLaunchKernelGGL(kvc_quant_channel_once_kernel, grid, dim3(KVC_WG), 0, stream, a);
+        else if (wide) hipLaunchKernelGGL(kvc_quant_channel8_kernel, grid, dim3(KVC_WG), 0, stream, a);
         else hipLaunchKernelGGL(kvc_quant_channel_kernel, grid, dim3(KVC_WG), 0, stream, a);
     } else if (quant_mask == KVC_MASK_V_TOKEN || quant_mask == KVC_MASK_SIM_TOKEN || quant_mask == KVC_MASK_VECTOR) {
         const int64_t R = quant_mask == KVC_MASK_V_TOKEN ? stride : quant_mask == KVC_MASK_SIM_TOKEN ? H * D : D;
         const int64_t groups = NB * BS * stride / R;
         const int wide = R % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
-        hipLaunchKernelGGL(kvc_quant_row_kernel, dim3((unsigned)((groups + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG)),
-                           dim3(KVC_WG), 0, stream, a, R, groups, wide);
+        const dim3 grid((unsigned)((groups + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG));
+        const bool once = wide && a.sym != nullptr && a.xhat == nullptr && R >= 512;    // the row fits a wave's registers
+        if (once && R <= 512 * 8) hipLaunchKernelGGL(kvc_quant_row_once_kernel<8>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
+        else if (once && R <= 512 * 16) hipLaunchKernelGGL(kvc_quant_row_once_kernel<16>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
+        else if (once && R <= 512 * 24) hipLaunchKernelGGL(kvc_quant_row_once_kernel<24>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
+        else if (once && R <= 512 * 32) hipLaunchKernelGGL(kvc_quant_row_once_kernel<32>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
+        else hipLaunchKernelGGL(kvc_quant_row_kernel, grid, dim3(KVC_WG), 0, stream, a, R, groups, wide);
     } else if (quant_mask == KVC_MASK_K_BLOCK || quant_mask == KVC_MASK_SIM_BLOCK) {
         const int64_t R = quant_mask == KVC_MASK_K_BLOCK ? stride : H * D;
         const int64_t rows = NB * BS * stride / R;

@@ -172,6 +172,15 @@ def test_quant_narrow_rows_bit_exact(mask):
     _quant_dequant_case(mask, 0.1, geometry=(128, 1, 3, 6))
 
 
+@pytest.mark.parametrize("geometry", [(128, 1, 48, 128), (128, 3, 4, 72), (64, 1, 96, 128), (64, 1, 100, 128), (64, 1, 130, 128)])
+def test_quant_rows_kept_in_registers_bit_exact(geometry):
+    """Per-token rows of 512 to 16 384 elements are read once and kept in the wave's registers (8, 16, 24 or 32 chunks
+    of 16 bytes per lane: rows of 6144, 864 -- whose last chunk only some lanes hold --, 12 288 and 12 800 elements),
+    longer ones (16 640) are read twice; per-channel blocks of 64 tokens are kept in registers at any width."""
+    for mask in (O.MASK_V_TOKEN, O.MASK_CHANNEL):
+        _quant_dequant_case(mask, 0.1, geometry=geometry)
+
+
 def _quant_dequant_case(mask, eb, geometry=(256, 2, 4, 128)):
     from kvcomp_amd import compute as cp
     T, B, H, D = geometry
