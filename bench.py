@@ -361,10 +361,26 @@ def other_configs(args):
                               "steps": loop["steps"], "compression_ratio_whole_cache": loop["config"]["compression_ratio_whole_cache"],
                               "prefill_compress_s": loop["config"]["prefill_compress_s"], "not_run": loop["config"]["not_run"]}
     log("[bench] cfg4 cache loop: %.2f ms per step, %.0f tokens/s" % (loop["ms_per_step"], loop["value"]))
+    # cfg4 with the model around the cache (random weights), and the same model on transformers' dense fp16 cache
+    try:
+        import transformers  # noqa: F401
+    except ImportError:
+        res["cfg4_model"] = None
+        return res
+    model = {}
+    for key, dense in (("compressed_cache", False), ("dense_fp16_cache", True)):
+        r = run_model_decode(types.SimpleNamespace(model_layers=32, new_tokens=64, warmup=5, dense_cache=dense), emit=False)
+        model[key] = {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
+                      "prefill_s": r["config"]["prefill_s"], "cache_bytes_held": r["config"]["cache_bytes_held"],
+                      "compression_ratio_whole_cache": r["config"]["compression_ratio_whole_cache"],
+                      "attention": r["config"]["attention"]}
+        log("[bench] cfg4 model, %s: %.2f ms per step, %.0f tokens/s" % (key.replace("_", " "), r["ms_per_step"], r["value"]))
+    model["workload"] = "Llama-2-7B architecture (stock transformers code, random fp16 weights), 32 layers, batch 8, 4096-token random prompt, 64 greedy tokens"
+    res["cfg4_model"] = model
     return res
 
 
-def run_model_decode(args):
+def run_model_decode(args, emit=True):
     """cfg4 as BASELINE.json words it: the Llama-2-7B architecture with random-init fp16 weights (stock `transformers`
     modelling code), a compressed KV cache in every layer, batch 8, a 4096-token random prompt and greedy generation;
     single-token steps attend on the compressed form through the "kvcomp" attention implementation.  Tokens are random,
@@ -432,7 +448,11 @@ def run_model_decode(args):
                                  "single-token steps: kvc_attention_decode on the compressed streams; prompt: stock SDPA")},
         "roofline": None, "cpu_baseline": None,
     }
-    print(json.dumps(result), flush=True)
+    if emit:
+        print(json.dumps(result), flush=True)
+    del model, cache, logits, nxt
+    torch.cuda.empty_cache()
+    return result
 
 
 def main():
