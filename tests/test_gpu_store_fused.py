@@ -310,3 +310,33 @@ def test_one_pass_and_two_pass_encoders_write_the_same_bytes(is_k, D, dist, one_
     pay, bi, ti = O.encode_tiles(o[3], is_k, f1.encode_codebook.cpu().numpy(), 0, vec_len=D if is_k else 128)
     assert np.array_equal(f1.encoded_data.cpu().numpy()[:pay.size], pay)
     assert np.array_equal(f1.block_infos.cpu().numpy()[:bi.size], bi)
+
+
+@pytest.mark.parametrize("is_k,T,B,H,D", [(True, 64 * 7, 1, 9, 96), (True, 64 * 19, 3, 1, 128), (False, 128 * 21, 1, 2, 96),
+                                          (False, 128 * 57, 1, 1, 64)])
+def test_one_pass_runs_of_two_over_odd_tile_counts(is_k, T, B, H, D):
+    """Two tiles per wave forced on streams of 63, 57, 63 and 57 tiles: the last wave holds a single tile, which also
+    closes the last (short) group of tiles; the first group is a full one of 56.  Payload and metadata must be the
+    oracle's, and a second store must continue behind the first."""
+    from kvcomp_amd import _lib
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    eb = 0.1 if is_k else 0.2
+    x = _data(is_k, T, B, H, D, "gauss", 31).to(DEV)
+    was = _lib.set_option("encode_one_pass", 3)
+    try:
+        ctx = KVCompCtx(is_k, B, H, D, eb)
+        ctx.build_codebook([x])
+        ctx.store(x, want_symbols=False)
+        ctx.store(x, want_symbols=False)
+    finally:
+        _lib.set_option("encode_one_pass", was)
+    o = O.quant(S.np16(S.blocked(x.cpu(), ctx.block_size)), _oracle_mask(ctx), eb)
+    pay, bi, ti = O.encode_tiles(o[3], is_k, ctx.encode_codebook.cpu().numpy(), 0, vec_len=D if is_k else 128)
+    assert bi.size // 8 in (57, 63)
+    got_bi, got_ti, got = ctx.block_infos.cpu().numpy(), ctx.thread_infos.cpu().numpy(), ctx.encoded_data.cpu().numpy()
+    assert np.array_equal(got_bi[:bi.size], bi) and np.array_equal(got_ti[:ti.size], ti)
+    assert np.array_equal(got[:pay.size], pay) and np.array_equal(got[pay.size:2 * pay.size], pay)
+    second = got_bi[bi.size:2 * bi.size].view(np.uint32).reshape(-1, 2)
+    first = bi.view(np.uint32).reshape(-1, 2)
+    assert np.array_equal(second[:, 0], first[:, 0] + pay.size) and np.array_equal(second[:, 1], first[:, 1])
