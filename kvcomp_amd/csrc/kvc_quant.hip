@@ -181,7 +181,29 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel8_kernel(KvcQuantArgs
         kvc_quant_store8<1>(a, base + t * stride, *reinterpret_cast<const uint4 *>(p + t * stride), gp);
 }
 
-// Per-channel groups over blocks of 64 tokens, symbols (and parameters) out: a thread keeps its two channels of all
+// The simulated-quantization values of two elements from kvc_quant_pair_biased's result: u - 1024 is the fp16 symbol the
+// reference keeps un-cast (rint(x / scale) - min, exact), then its two fp16 tensor ops (utils/compute.py:130):
+// (symbol + min) -- the sum of two integers, exact -- times scale, one rounding.
+__device__ __forceinline__ uint32_t kvc_quant_error_pair(uint32_t u, uint32_t min2, uint32_t scale2)
+{
+#pragma clang fp contract(off)
+    const kvc_half2 bias = {(_Float16)1024.f, (_Float16)1024.f};
+    const kvc_half2 sym = __builtin_bit_cast(kvc_half2, u) - bias;
+    const kvc_half2 v = (sym + __builtin_bit_cast(kvc_half2, min2)) * __builtin_bit_cast(kvc_half2, scale2);
+    return __builtin_bit_cast(uint32_t, v);
+}
+// kvc_quant_pair_biased gives the reference's integers where every quotient x / scale of the group stays within +-512
+// (kvc_quant_math.h); the group's smallest and largest quotients say whether it does (false for a zero scale too).
+__device__ __forceinline__ bool kvc_packed_quantizer_applies(const KvcGroupParams &g, float mx)
+{
+    return fabsf(g.min_i) <= 500.f && fabsf(mx * g.rcp) <= 500.f;
+}
+__device__ __forceinline__ uint32_t kvc_half_pair_bits(__half lo, __half hi)
+{
+    return (uint32_t)__half_as_ushort(lo) | ((uint32_t)__half_as_ushort(hi) << 16);
+}
+
+// Per-channel groups over blocks of 64 tokens, symbols and / or simulated-quantization values out: a thread keeps its two channels of all
 // 64 tokens in registers, so the block is read once (64 loads in flight), finds minima and maxima with packed fp16
 // min / max and quantizes two channels per instruction (kvc_quant_pair_biased: the same symbols as the fp32 chain for
 // every fp16 input, see kvc_quant_math.h).
@@ -210,12 +232,18 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_channel_once_kernel(KvcQuant
     const int64_t g = nb * stride + c;
     kvc_quant_publish(a, g, g0);
     kvc_quant_publish(a, g + 1, g1);
-    const KvcPackedParams pp = kvc_packed_params(g0, g1);
-    uint8_t *out = a.sym + base;
+    if (kvc_packed_quantizer_applies(g0, kvc_half_lo(mxw)) && kvc_packed_quantizer_applies(g1, kvc_half_hi(mxw))) {
+        const KvcPackedParams pp = kvc_packed_params(g0, g1);
+        const uint32_t min2 = kvc_half_pair_bits(g0.min_h, g1.min_h), scale2 = kvc_half_pair_bits(g0.scale_h, g1.scale_h);
 #pragma unroll
-    for (int t = 0; t < KVC_WAVE; t++) {
-        const uint32_t u = kvc_quant_pair_biased(raw[t], pp);
-        *reinterpret_cast<uint16_t *>(out + t * stride) = (uint16_t)kvc_low_bytes4(u, u);
+        for (int t = 0; t < KVC_WAVE; t++) {
+            const uint32_t u = kvc_quant_pair_biased(raw[t], pp);
+            if (a.sym) *reinterpret_cast<uint16_t *>(a.sym + base + t * stride) = (uint16_t)kvc_low_bytes4(u, u);
+            if (a.xhat) *reinterpret_cast<uint32_t *>(a.xhat + base + t * stride) = kvc_quant_error_pair(u, min2, scale2);
+        }
+    } else {                                               // quotients beyond the packed arithmetic's range, or a zero scale
+#pragma unroll                                             // (fully: a run-time index would move the block out of the registers)
+        for (int t = 0; t < KVC_WAVE; t++) kvc_quant_store2(a, base + t * stride, kvc_half_lo(raw[t]), kvc_half_hi(raw[t]), g0, g1);
     }
 }
 
@@ -253,7 +281,8 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_kernel(KvcQuantArgs a, i
     }
 }
 
-// Row groups of 512 to 512 NIT elements (a multiple of 8, 16-byte aligned buffers), symbols (and parameters) out: the
+// Row groups of 512 to 512 NIT elements (a multiple of 8, 16-byte aligned buffers), symbols and / or simulated-quantization
+// values out: the
 // wave keeps the row in registers (NIT 16-byte loads per lane in flight), so it is read once, and quantizes two
 // elements per instruction (kvc_quant_pair_biased, as the per-channel kernel above).
 template <int NIT>
@@ -297,15 +326,26 @@ __global__ void __launch_bounds__(KVC_WG) kvc_quant_row_once_kernel(KvcQuantArgs
     const float hi = kvc_wave_max(fmaxf(kvc_half_lo(mxw), kvc_half_hi(mxw)));
     const KvcGroupParams gp = kvc_group_params(lo, hi, a.eb);
     if (lane == 0) kvc_quant_publish(a, g, gp);
+    if (!kvc_packed_quantizer_applies(gp, hi)) {           // (wave-uniform) quotients beyond the packed arithmetic's range, or a zero scale
+#pragma unroll
+        for (int j = 0; j < NIT; j++) {
+            const int64_t i = 8 * lane + 512 * j;
+            if (i < R) kvc_quant_store8<0>(a, g * R + i, raw[j], &gp);
+        }
+        return;
+    }
     const KvcPackedParams pp = kvc_packed_params(gp, gp);
-    uint8_t *out = a.sym + g * R;
+    const uint32_t min2 = kvc_half_pair_bits(gp.min_h, gp.min_h), scale2 = kvc_half_pair_bits(gp.scale_h, gp.scale_h);
 #pragma unroll
     for (int j = 0; j < NIT; j++) {
         const int64_t i = 8 * lane + 512 * j;
         if (i < R) {
             const uint32_t u0 = kvc_quant_pair_biased(raw[j].x, pp), u1 = kvc_quant_pair_biased(raw[j].y, pp);
             const uint32_t u2 = kvc_quant_pair_biased(raw[j].z, pp), u3 = kvc_quant_pair_biased(raw[j].w, pp);
-            *reinterpret_cast<uint2 *>(out + i) = make_uint2(kvc_low_bytes4(u0, u1), kvc_low_bytes4(u2, u3));
+            if (a.sym) *reinterpret_cast<uint2 *>(a.sym + g * R + i) = make_uint2(kvc_low_bytes4(u0, u1), kvc_low_bytes4(u2, u3));
+            if (a.xhat)
+                *reinterpret_cast<uint4 *>(a.xhat + g * R + i) = make_uint4(kvc_quant_error_pair(u0, min2, scale2), kvc_quant_error_pair(u1, min2, scale2),
+                                                                           kvc_quant_error_pair(u2, min2, scale2), kvc_quant_error_pair(u3, min2, scale2));
         }
     }
 }
@@ -397,7 +437,7 @@ static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t
     const int64_t stride = B * H * D;
     if (quant_mask == KVC_MASK_CHANNEL) {
         const bool wide = stride % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
-        const bool once = BS == KVC_WAVE && a.sym != nullptr && a.xhat == nullptr;     // the block fits a thread's registers
+        const bool once = BS == KVC_WAVE && (a.sym != nullptr || a.xhat != nullptr);   // the block fits a thread's registers
         const int64_t threads = NB * (once || !wide ? stride / 2 : stride / 8);
         const dim3 grid((unsigned)((threads + KVC_WG - 1) / KVC_WG));
         if (once) hipLaunchKernelGGL(kvc_quant_channel_once_kernel, grid, dim3(KVC_WG), 0, stream, a);
@@ -408,7 +448,7 @@ static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t
         const int64_t groups = NB * BS * stride / R;
         const int wide = R % 8 == 0 && ((uintptr_t)a.x & 15) == 0 && ((uintptr_t)a.sym & 7) == 0 && ((uintptr_t)a.xhat & 15) == 0;
         const dim3 grid((unsigned)((groups + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG));
-        const bool once = wide && a.sym != nullptr && a.xhat == nullptr && R >= 512;    // the row fits a wave's registers
+        const bool once = wide && (a.sym != nullptr || a.xhat != nullptr) && R >= 512;  // the row fits a wave's registers
         if (once && R <= 512 * 8) hipLaunchKernelGGL(kvc_quant_row_once_kernel<8>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
         else if (once && R <= 512 * 16) hipLaunchKernelGGL(kvc_quant_row_once_kernel<16>, grid, dim3(KVC_WG), 0, stream, a, R, groups);
         else if (once && R <= 512 * 24) hipLaunchKernelGGL(kvc_quant_row_once_kernel<24>, grid, dim3(KVC_WG), 0, stream, a, R, groups);

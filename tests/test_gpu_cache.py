@@ -73,14 +73,17 @@ def test_quant_dequant_sim_is_bit_exact(mode):
     assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
 
 
-def test_quant_dequant_sim_keeps_minima_outside_int8():
-    """Channels that sit far from zero relative to their range have min/scale beyond +-127; the sim path keeps
-    them as fp16 numbers (the entropy-coded path would wrap them into int8)."""
+@pytest.mark.parametrize("mode,offset", [("ChannelQuant", 40.0), ("TokenQuant", 40.0), ("ChannelQuant", 12.0), ("TokenQuant", 12.0)])
+def test_quant_dequant_sim_keeps_minima_outside_int8(mode, offset):
+    """Groups that sit far from zero relative to their range have min/scale beyond +-127 (about 800 and 240 here); the
+    sim path keeps them as fp16 numbers (the entropy-coded path would wrap them into int8).  Quotients beyond +-512
+    are also outside what the two-elements-per-instruction quantizer covers: those groups take the fp32 chain, the
+    ones at 240 the packed arithmetic (rows of 512 elements and 64-token blocks are kept in registers either way)."""
     from kvcomp_amd.compute import QuantMode, quant_dequant_sim
     g = torch.Generator().manual_seed(5)
-    x = (torch.rand(1, 2, 128, 64, generator=g) * 0.5 + 40.0).to(torch.float16)       # min/scale ~ 800
-    got = quant_dequant_sim(x.to(DEV), 64, 0.1, QuantMode.ChannelQuant).cpu()
-    ref = _sim_cpu(x, 64, 0.1, "ChannelQuant")
+    x = (torch.rand(1, 8, 128, 64, generator=g) * 0.5 + offset).to(torch.float16)
+    got = quant_dequant_sim(x.to(DEV), 64, 0.1, QuantMode(mode)).cpu()
+    ref = _sim_cpu(x, 64, 0.1, mode)
     assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
     assert (got.float() - x.float()).abs().max() < 0.1
 
