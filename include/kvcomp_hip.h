@@ -88,7 +88,7 @@ int kvc_abi_version(void);
  *                           for the first p %, r / 2 for the next q %, r / 4 and 1 for halves of the rest.
  *   "encode_one_pass":       1 (default): the fused quantize + encode (kvc_store_fused, kvc_encode_async from fp16) reads
  *                           its input once: a wave quantizes and counts its tiles, finds their place in the payload by looking back
- *                           over the sizes the tiles before it have published, and emits them; so do K encodes from uint8
+ *                           over the sizes the tiles before it have published, and emits them; so do encodes from uint8
  *                           symbols of at least 8192 tiles.  0: two passes (count, offsets, emit), also taken when
  *                           block_infos is not 8-byte aligned or the call has more than 84 224 tiles, and by the other
  *                           encoders that start from uint8 symbols; 2 / 3: one pass for every encoder, with

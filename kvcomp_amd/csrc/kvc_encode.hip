@@ -125,6 +125,43 @@ __device__ __forceinline__ void kvc_load_vector(const KvcEncodeArgs &a, int64_t 
     }
 }
 
+// The same vectors of a V tile fetched four channels per lane: 16 lanes cover a token's 64 symbols, a load instruction
+// four tokens (the byte-per-token-row loads above move 64 bytes per instruction, 128 instructions per tile; these move
+// 256 bytes, 32 instructions), four tokens of four channels are transposed in registers and go to the wave's LDS tile
+// as [channel][token], and lane c then reads channel c's vector.  Needs the row stride to be a multiple of 4 and the
+// symbols 4-byte aligned (every encode call is checked for that).
+__device__ __forceinline__ void kvc_load_vector_v_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_tile, uint32_t v[32])
+{
+    constexpr int RS = KVC_V_TOKENS + 4;
+    const int64_t row = tile / a.cols, col = tile - row * a.cols;
+    const int pr = lane & 15, sub = lane >> 4;
+    const uint8_t *p = a.sym + (row * KVC_V_TOKENS + 4 * sub) * a.stride + col * KVC_WAVE + 4 * pr;
+    uint32_t w[32];
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++)
+#pragma unroll
+        for (int k = 0; k < 4; k++) w[4 * jj + k] = *reinterpret_cast<const uint32_t *>(p + (int64_t)(16 * jj + k) * a.stride);
+#pragma unroll
+    for (int jj = 0; jj < 8; jj++) {
+        const uint32_t w0 = w[4 * jj], w1 = w[4 * jj + 1], w2 = w[4 * jj + 2], w3 = w[4 * jj + 3];
+        // {w0.b0 w1.b0 w0.b1 w1.b1}, {w0.b2 w1.b2 w0.b3 w1.b3}, the same of w2 and w3; then a channel's four tokens
+        const uint32_t a_lo = __builtin_amdgcn_perm(w1, w0, 0x05010400u), a_hi = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
+        const uint32_t b_lo = __builtin_amdgcn_perm(w3, w2, 0x05010400u), b_hi = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
+        const uint32_t c0 = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u), c1 = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
+        const uint32_t c2 = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u), c3 = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
+        uint8_t *dst = s_tile + (4 * pr) * RS + 16 * jj + 4 * sub;
+        *reinterpret_cast<uint32_t *>(dst) = c0;
+        *reinterpret_cast<uint32_t *>(dst + RS) = c1;
+        *reinterpret_cast<uint32_t *>(dst + 2 * RS) = c2;
+        *reinterpret_cast<uint32_t *>(dst + 3 * RS) = c3;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = *reinterpret_cast<const uint32_t *>(s_tile + lane * RS + 4 * j);
+}
+
 // What the count step of one tile finds out (every field wave-uniform except `start`).
 struct KvcTileCount {
     uint32_t start;      // first byte of this lane's stream inside the tile payload
@@ -1000,7 +1037,8 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
             kvc_front_v(a, tile, lane, s_sym, s_par, raw, v);
             if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_v_load(a, tile + 1, lane, raw);
         } else {
-            kvc_load_vector(a.e, tile, lane, v);
+            if (a.e.is_k) kvc_load_vector(a.e, tile, lane, v);
+            else kvc_load_vector_v_tile(a.e, tile, lane, s_sym, v);       // (the launcher requires 4-byte aligned symbols and rows)
         }
         kvc_wave_lds_sync();                               // every lane holds its vector: the tile area is free
         uint32_t bits = 0;
@@ -1212,10 +1250,11 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     hipLaunchKernelGGL(kvc_encode_init_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
     // one pass (each wave counts, places and emits its tile) where the block_infos can serve as 64-bit status words.
     // From uint8 symbols there is no quantizing to save and the one-pass kernel runs at three waves per SIMD: measured on
-    // MI355X at 65 536 tiles, K symbols encode 1.17 times faster in one pass and V symbols 1.4 times faster in two, so
-    // by default only large K calls take the one pass (the option's values 2 and 3 send every call through it).
+    // MI355X at 65 536 / 49 152 tiles, K symbols encode 1.17 times and V symbols (which the one-pass kernel fetches four
+    // channels per lane through its LDS tile) 1.6 times faster in one pass than in two.  So by default large calls
+    // take the one pass (the option's values 2 and 3 send every call through it).
     const int one_pass = kvc_option(KVC_OPT_ENCODE_ONE_PASS);
-    const bool symbols_in_one_pass = one_pass > 1 || (one_pass == 1 && is_k && a.tiles >= 8192);
+    const bool symbols_in_one_pass = one_pass > 1 || (one_pass == 1 && a.tiles >= 8192);
     if ((src ? one_pass != 0 : symbols_in_one_pass) && ((uintptr_t)c.d_block_infos & 7) == 0 &&
         (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES <= KVC_ONCE_MAX_GROUPS) {
         if (!src) sa.e = a;
