@@ -162,6 +162,33 @@ __device__ __forceinline__ void kvc_load_vector_v_tile(const KvcEncodeArgs &a, i
     for (int j = 0; j < 32; j++) v[j] = *reinterpret_cast<const uint32_t *>(s_tile + lane * RS + 4 * j);
 }
 
+// K vectors through the LDS tile as well: vec_len / 4 lanes cover a token's run, a load instruction two or more tokens
+// (with a token per lane, as above, every instruction touches 64 rows of the symbol tensor), the words go to the tile
+// as [token][channel] with rows vec_len + 4 bytes apart, and lane t then reads token t's row.  vec_len <= 128.
+__device__ __forceinline__ void kvc_load_vector_k_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_tile, uint32_t v[32])
+{
+    const int64_t row = tile / a.cols, col = tile - row * a.cols;
+    const int nd = a.vec_len >> 2, RS = a.vec_len + 4;
+    const int per = KVC_WAVE / nd;                                     // tokens per load instruction (at least 2)
+    const int r = lane / nd, cw = lane - r * nd;
+    const bool active = r < per;
+    const uint8_t *p = a.sym + (row * KVC_WAVE + r) * a.stride + col * a.vec_len + 4 * cw;
+    uint32_t w[32];
+#pragma unroll
+    for (int i = 0; i < 32; i++) {
+        w[i] = 0u;
+        if (active && r + per * i < KVC_WAVE) w[i] = *reinterpret_cast<const uint32_t *>(p + (int64_t)(per * i) * a.stride);
+    }
+#pragma unroll
+    for (int i = 0; i < 32; i++)
+        if (active && r + per * i < KVC_WAVE) *reinterpret_cast<uint32_t *>(s_tile + (r + per * i) * RS + 4 * cw) = w[i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_tile + lane * RS + 4 * j) : 0u;
+}
+
 // What the count step of one tile finds out (every field wave-uniform except `start`).
 struct KvcTileCount {
     uint32_t start;      // first byte of this lane's stream inside the tile payload
@@ -1037,7 +1064,7 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
             kvc_front_v(a, tile, lane, s_sym, s_par, raw, v);
             if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_v_load(a, tile + 1, lane, raw);
         } else {
-            if (a.e.is_k) kvc_load_vector(a.e, tile, lane, v);
+            if (a.e.is_k) kvc_load_vector_k_tile(a.e, tile, lane, s_sym, v);
             else kvc_load_vector_v_tile(a.e, tile, lane, s_sym, v);       // (the launcher requires 4-byte aligned symbols and rows)
         }
         kvc_wave_lds_sync();                               // every lane holds its vector: the tile area is free
@@ -1250,9 +1277,9 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     hipLaunchKernelGGL(kvc_encode_init_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
     // one pass (each wave counts, places and emits its tile) where the block_infos can serve as 64-bit status words.
     // From uint8 symbols there is no quantizing to save and the one-pass kernel runs at three waves per SIMD: measured on
-    // MI355X at 65 536 / 49 152 tiles, K symbols encode 1.17 times and V symbols (which the one-pass kernel fetches four
-    // channels per lane through its LDS tile) 1.6 times faster in one pass than in two.  So by default large calls
-    // take the one pass (the option's values 2 and 3 send every call through it).
+    // MI355X at 65 536 / 49 152 tiles, K symbols encode 1.5 times and V symbols 1.6 times faster in one pass (which
+    // fetches them through its LDS tile, whole token rows per load instruction) than in two.  So by default large
+    // calls take the one pass (the option's values 2 and 3 send every call through it).
     const int one_pass = kvc_option(KVC_OPT_ENCODE_ONE_PASS);
     const bool symbols_in_one_pass = one_pass > 1 || (one_pass == 1 && a.tiles >= 8192);
     if ((src ? one_pass != 0 : symbols_in_one_pass) && ((uintptr_t)c.d_block_infos & 7) == 0 &&

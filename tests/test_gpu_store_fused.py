@@ -312,12 +312,14 @@ def test_one_pass_and_two_pass_encoders_write_the_same_bytes(is_k, D, dist, one_
     assert np.array_equal(f1.block_infos.cpu().numpy()[:bi.size], bi)
 
 
+@pytest.mark.parametrize("from_symbols", [False, True])
 @pytest.mark.parametrize("is_k,T,B,H,D", [(True, 64 * 7, 1, 9, 96), (True, 64 * 19, 3, 1, 128), (False, 128 * 21, 1, 2, 96),
-                                          (False, 128 * 57, 1, 1, 64)])
-def test_one_pass_runs_of_two_over_odd_tile_counts(is_k, T, B, H, D):
-    """Two tiles per wave forced on streams of 63, 57, 63 and 57 tiles: the last wave holds a single tile, which also
-    closes the last (short) group of tiles; the first group is a full one of 56.  Payload and metadata must be the
-    oracle's, and a second store must continue behind the first."""
+                                          (False, 128 * 57, 1, 1, 64), (True, 64 * 3, 3, 7, 72), (True, 64 * 9, 1, 7, 40)])
+def test_one_pass_runs_of_two_over_odd_tile_counts(is_k, T, B, H, D, from_symbols):
+    """Two tiles per wave forced on streams of 63 and 57 tiles: the last wave holds a single tile, which also
+    closes the last (short) group of tiles; the first group is a full one of 56.  From fp16 and from uint8 symbols
+    (which the one-pass kernel fetches through its LDS tile: head sizes whose words do not divide the 64 lanes
+    included).  Payload and metadata must be the oracle's, and a second store must continue behind the first."""
     from kvcomp_amd import _lib
     from kvcomp_amd.ctx import KVCompCtx
     _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
@@ -327,8 +329,8 @@ def test_one_pass_runs_of_two_over_odd_tile_counts(is_k, T, B, H, D):
     try:
         ctx = KVCompCtx(is_k, B, H, D, eb)
         ctx.build_codebook([x])
-        ctx.store(x, want_symbols=False)
-        ctx.store(x, want_symbols=False)
+        ctx.store(x, want_symbols=from_symbols)
+        ctx.store(x, want_symbols=from_symbols)
     finally:
         _lib.set_option("encode_one_pass", was)
     o = O.quant(S.np16(S.blocked(x.cpu(), ctx.block_size)), _oracle_mask(ctx), eb)
