@@ -111,16 +111,17 @@ class CompressedAttention:
         d = _lib.CompressedDesc()
         if ctx.compressed_ctx_len:
             d.d_luts = lut.data_ptr()
-            d.d_block_infos, d.block_infos_bytes = ctx.block_infos.data_ptr(), ctx.block_infos.numel()
-            d.d_thread_infos, d.thread_infos_bytes = ctx.thread_infos.data_ptr(), ctx.thread_infos.numel()
+            # (addresses and sizes straight from the contexts' growing arrays: a tensor view per field and call costs more
+            # host time than a short-context step takes on the device)
+            d.d_block_infos, d.block_infos_bytes = ctx._block_infos.address_and_numel()
+            d.d_thread_infos, d.thread_infos_bytes = ctx._thread_infos.address_and_numel()
             enc, enc_bytes = ctx.encoded_nosync()          # an address and a bound: no wait for queued encodes
             d.d_encoded, d.encoded_bytes = enc.data_ptr(), enc_bytes
             # the kernels take the quantization parameters by pointer: they must cover every group of the stream
             groups = expected_groups(ctx.compressed_ctx_len, ctx.block_size, ctx.batch_size, ctx.head_num, ctx.head_dim, ctx.quant_dims)
-            assert ctx.quant_min_ints.numel() == groups and ctx.quant_scales.numel() == groups, \
-                "the context holds %d minima and %d scales for %d quantization groups" % (
-                    ctx.quant_min_ints.numel(), ctx.quant_scales.numel(), groups)
-            d.d_quant_min_ints, d.d_quant_scales_f16 = ctx.quant_min_ints.data_ptr(), ctx.quant_scales.data_ptr()
+            (d.d_quant_min_ints, n_min), (d.d_quant_scales_f16, n_scale) = ctx._min_ints.address_and_numel(), ctx._scales.address_and_numel()
+            assert n_min == groups and n_scale == groups, \
+                "the context holds %d minima and %d scales for %d quantization groups" % (n_min, n_scale, groups)
         d.rows_per_codebook = 0
         d.quant_mask = dims_to_mask(ctx.quant_dims)
         d.max_tile_bytes, d.max_stream_bytes, d.max_code_bits = ctx.max_tile_bytes, ctx.max_stream_bytes, ctx.max_code_bits

@@ -146,6 +146,15 @@ class _Growable:
     def view(self) -> Optional[torch.Tensor]:
         return None if self.data is None else self.data[:self.used]
 
+    def address_and_numel(self):
+        """(device address, elements) of the filled part without making a tensor for it (0, 0 while empty)."""
+        if self.data is None:
+            return 0, 0
+        row = 1
+        for n in self.data.shape[1:]:
+            row *= n
+        return self.data.data_ptr(), self.used * row
+
 
 class KVCompCtx:
     """One compressed K or V stream of one layer (models/cache/kvcomp_encode.py:15-326)."""
