@@ -51,6 +51,9 @@ struct KvcEncodeArgs {
     // results left on the device (kvc_encode_async): see kvc_encode_job in include/kvcomp_hip.h
     uint32_t *stream_bytes;    // NULL, or in / out: payload bytes already in `encoded`; this call appends behind them
     uint32_t *result;          // NULL, or uint32[8]
+    // one pass only: how often a wave may find a word of its look-back not ready before it gives up, and whether the
+    // call is to be treated as if a wave had given up (both from the option "encode_lookback_polls")
+    int max_polls, force_order;
 };
 
 constexpr int KVC_ENC_STATUS_WORDS = 16;            // status words in front of the per-1024-tile payload totals
@@ -98,6 +101,7 @@ __global__ void kvc_encode_publish_kernel(KvcEncodeArgs a)
         if (a.status[3] > a.result[3]) a.result[3] = a.status[3];
         a.result[4] += (uint32_t)a.tiles;
         a.result[5] = a.status[KVC_ENC_ST_BASE];
+        if (a.status[6] > a.result[6]) a.result[6] = a.status[6];
     }
     if (a.stream_bytes && !err) *a.stream_bytes = a.status[KVC_ENC_ST_BASE] - a.base_global_offset + total;
 }
@@ -125,14 +129,32 @@ __device__ __forceinline__ void kvc_load_vector(const KvcEncodeArgs &a, int64_t 
     }
 }
 
+// LDS traffic between the lanes of one wave needs no workgroup barrier (a wave's LDS operations complete in
+// order); this keeps the compiler from moving accesses across the hand-over.
+__device__ __forceinline__ void kvc_wave_lds_sync()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// A tile's symbols change hands between lanes through a staging area in LDS (the lane that loads or quantizes a symbol
+// is not the lane whose vector it belongs to).  The area holds a part of the tile at a time -- half of it, or a quarter
+// where V is quantized from fp16 -- so that, in the one-pass kernel, a payload of any size (up to KVC_MAX_TILE_BYTES)
+// can wait in the same wave's LDS while the next tile is staged.
+constexpr int KVC_STAGE_K_BYTES = 32 * (128 + 4);       // 32 tokens of up to 128 symbols, rows 4 bytes apart from a multiple of 128 (from
+                                                        // symbols: also 48 tokens of at most 80 symbols, 64 of at most 64)
+constexpr int KVC_STAGE_VSYM_BYTES = 64 * (64 + 4);     // 64 channels of 64 tokens
+constexpr int KVC_STAGE_VF16_BYTES = 64 * (32 + 4);     // 64 channels of 32 tokens
+
 // The same vectors of a V tile fetched four channels per lane: 16 lanes cover a token's 64 symbols, a load instruction
 // four tokens (the byte-per-token-row loads above move 64 bytes per instruction, 128 instructions per tile; these move
-// 256 bytes, 32 instructions), four tokens of four channels are transposed in registers and go to the wave's LDS tile
-// as [channel][token], and lane c then reads channel c's vector.  Needs the row stride to be a multiple of 4 and the
-// symbols 4-byte aligned (every encode call is checked for that).
-__device__ __forceinline__ void kvc_load_vector_v_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_tile, uint32_t v[32])
+// 256 bytes, 32 instructions), four tokens of four channels are transposed in registers and go to the staging area
+// as [channel][token], 64 tokens at a time, and lane c then reads channel c's vector.  Needs the row stride to be a
+// multiple of 4 and the symbols 4-byte aligned (every encode call is checked for that).
+__device__ __forceinline__ void kvc_load_vector_v_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_stage, uint32_t v[32])
 {
-    constexpr int RS = KVC_V_TOKENS + 4;
+    constexpr int RS = 64 + 4;
     const int64_t row = tile / a.cols, col = tile - row * a.cols;
     const int pr = lane & 15, sub = lane >> 4;
     const uint8_t *p = a.sym + (row * KVC_V_TOKENS + 4 * sub) * a.stride + col * KVC_WAVE + 4 * pr;
@@ -142,30 +164,44 @@ __device__ __forceinline__ void kvc_load_vector_v_tile(const KvcEncodeArgs &a, i
 #pragma unroll
         for (int k = 0; k < 4; k++) w[4 * jj + k] = *reinterpret_cast<const uint32_t *>(p + (int64_t)(16 * jj + k) * a.stride);
 #pragma unroll
-    for (int jj = 0; jj < 8; jj++) {
-        const uint32_t w0 = w[4 * jj], w1 = w[4 * jj + 1], w2 = w[4 * jj + 2], w3 = w[4 * jj + 3];
-        // {w0.b0 w1.b0 w0.b1 w1.b1}, {w0.b2 w1.b2 w0.b3 w1.b3}, the same of w2 and w3; then a channel's four tokens
-        const uint32_t a_lo = __builtin_amdgcn_perm(w1, w0, 0x05010400u), a_hi = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
-        const uint32_t b_lo = __builtin_amdgcn_perm(w3, w2, 0x05010400u), b_hi = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
-        const uint32_t c0 = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u), c1 = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
-        const uint32_t c2 = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u), c3 = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
-        uint8_t *dst = s_tile + (4 * pr) * RS + 16 * jj + 4 * sub;
-        *reinterpret_cast<uint32_t *>(dst) = c0;
-        *reinterpret_cast<uint32_t *>(dst + RS) = c1;
-        *reinterpret_cast<uint32_t *>(dst + 2 * RS) = c2;
-        *reinterpret_cast<uint32_t *>(dst + 3 * RS) = c3;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int h = 0; h < 2; h++) {
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = *reinterpret_cast<const uint32_t *>(s_tile + lane * RS + 4 * j);
+        for (int jj = 4 * h; jj < 4 * h + 4; jj++) {
+            const uint32_t w0 = w[4 * jj], w1 = w[4 * jj + 1], w2 = w[4 * jj + 2], w3 = w[4 * jj + 3];
+            // {w0.b0 w1.b0 w0.b1 w1.b1}, {w0.b2 w1.b2 w0.b3 w1.b3}, the same of w2 and w3; then a channel's four tokens
+            const uint32_t a_lo = __builtin_amdgcn_perm(w1, w0, 0x05010400u), a_hi = __builtin_amdgcn_perm(w1, w0, 0x07030602u);
+            const uint32_t b_lo = __builtin_amdgcn_perm(w3, w2, 0x05010400u), b_hi = __builtin_amdgcn_perm(w3, w2, 0x07030602u);
+            const uint32_t c0 = __builtin_amdgcn_perm(b_lo, a_lo, 0x05040100u), c1 = __builtin_amdgcn_perm(b_lo, a_lo, 0x07060302u);
+            const uint32_t c2 = __builtin_amdgcn_perm(b_hi, a_hi, 0x05040100u), c3 = __builtin_amdgcn_perm(b_hi, a_hi, 0x07060302u);
+            uint8_t *dst = s_stage + (4 * pr) * RS + 16 * (jj - 4 * h) + 4 * sub;
+            *reinterpret_cast<uint32_t *>(dst) = c0;
+            *reinterpret_cast<uint32_t *>(dst + RS) = c1;
+            *reinterpret_cast<uint32_t *>(dst + 2 * RS) = c2;
+            *reinterpret_cast<uint32_t *>(dst + 3 * RS) = c3;
+        }
+        kvc_wave_lds_sync();
+#pragma unroll
+        for (int j = 0; j < 16; j++) v[16 * h + j] = *reinterpret_cast<const uint32_t *>(s_stage + lane * RS + 4 * j);
+        kvc_wave_lds_sync();                                           // read: the area may take the next part
+    }
 }
 
-// K vectors through the LDS tile as well: vec_len / 4 lanes cover a token's run, a load instruction two or more tokens
-// (with a token per lane, as above, every instruction touches 64 rows of the symbol tensor), the words go to the tile
-// as [token][channel] with rows vec_len + 4 bytes apart, and lane t then reads token t's row.  vec_len <= 128.
-__device__ __forceinline__ void kvc_load_vector_k_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_tile, uint32_t v[32])
+// Token `lane`'s row of a K staging area that holds tokens 32 h .. 32 h + 31 (rows RS bytes apart).
+__device__ __forceinline__ void kvc_read_k_rows(const uint8_t *s_stage, int RS, int nd, int lane, int h, uint32_t (&v)[32])
+{
+    if ((lane >> 5) == h) {
+        const uint8_t *row = s_stage + (lane & 31) * RS;
+#pragma unroll
+        for (int j = 0; j < 32; j++)
+            if (j < nd) v[j] = *reinterpret_cast<const uint32_t *>(row + 4 * j);
+    }
+}
+
+// K vectors through the staging area as well: vec_len / 4 lanes cover a token's run, a load instruction two or more tokens
+// (with a token per lane, as above, every instruction touches 64 rows of the symbol tensor), the words go to the area
+// as [token][channel] with rows vec_len + 4 bytes apart, 32 tokens at a time, and lane t then reads token t's row.
+// vec_len <= 128.
+__device__ __forceinline__ void kvc_load_vector_k_tile(const KvcEncodeArgs &a, int64_t tile, int lane, uint8_t *s_stage, uint32_t (&v)[32])
 {
     const int64_t row = tile / a.cols, col = tile - row * a.cols;
     const int nd = a.vec_len >> 2, RS = a.vec_len + 4;
@@ -180,13 +216,26 @@ __device__ __forceinline__ void kvc_load_vector_k_tile(const KvcEncodeArgs &a, i
         if (active && r + per * i < KVC_WAVE) w[i] = *reinterpret_cast<const uint32_t *>(p + (int64_t)(per * i) * a.stride);
     }
 #pragma unroll
-    for (int i = 0; i < 32; i++)
-        if (active && r + per * i < KVC_WAVE) *reinterpret_cast<uint32_t *>(s_tile + (r + per * i) * RS + 4 * cw) = w[i];
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    for (int j = 0; j < 32; j++) v[j] = 0u;
+    // the first sixteen load instructions cover tokens 0 .. 16 per - 1 (all 64 where a token's run is at most 64 bytes),
+    // the other sixteen the rest: at most 32 tokens of 132 bytes, 48 of 84 or 64 of 68 in the area at a time
+    const int split = 16 * per;
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_tile + lane * RS + 4 * j) : 0u;
+    for (int h = 0; h < 2; h++) {
+        uint8_t *dst = s_stage + r * RS + 4 * cw;
+#pragma unroll
+        for (int i = 0; i < 16; i++)
+            if (active && r + per * (16 * h + i) < KVC_WAVE) *reinterpret_cast<uint32_t *>(dst + (per * i) * RS) = w[16 * h + i];
+        kvc_wave_lds_sync();
+        const int mine = lane - split * h;                 // this lane's row of the area, if it is in this part
+        if (mine >= 0 && (h == 1 || mine < split)) {
+            const uint8_t *rowp = s_stage + mine * RS;
+#pragma unroll
+            for (int j = 0; j < 32; j++)
+                if (j < nd) v[j] = *reinterpret_cast<const uint32_t *>(rowp + 4 * j);
+        }
+        kvc_wave_lds_sync();
+    }
 }
 
 // What the count step of one tile finds out (every field wave-uniform except `start`).
@@ -353,15 +402,6 @@ __global__ void __launch_bounds__(1024) kvc_encode_scan_kernel(KvcEncodeArgs a)
 
 constexpr int KVC_IMAGE_WORDS = (KVC_MAX_TILE_BYTES + 3 + 3) / 4 + 1;   // payload + up to 3 leading bytes
 
-// LDS traffic between the lanes of one wave needs no workgroup barrier (a wave's LDS operations complete in
-// order); this keeps the compiler from moving accesses across the hand-over.
-__device__ __forceinline__ void kvc_wave_lds_sync()
-{
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
 // Where tile `tile` goes: ok = it fits (a tile flagged by the earlier launches is skipped, never written out of bounds).
 struct KvcEmitPlace {
     uint32_t off, bn, head;
@@ -410,7 +450,8 @@ __device__ __forceinline__ uint32_t kvc_stream_start(const KvcEncodeArgs &a, int
 }
 
 __device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, uint32_t start, const uint32_t (&v)[32],
-                                                const uint2 *s_table, uint32_t *image, uint32_t head, bool short_codes)
+                                                const uint2 *s_table, uint32_t *image, uint32_t head, bool short_codes,
+                                                uint32_t image_words = (uint32_t)KVC_IMAGE_WORDS)
 {
     const uint32_t bitpos = (head + start) * 8u;
     uint32_t w = bitpos >> 5, nacc = bitpos & 31u;
@@ -421,7 +462,7 @@ __device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, uint32_t
         nacc += len;
         if (nacc >= 32u) {
             nacc -= 32u;
-            if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
+            if (w < image_words) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
             w++;
         }
     };
@@ -447,7 +488,7 @@ __device__ __forceinline__ void kvc_pack_vector(const KvcEncodeArgs &a, uint32_t
             }
         }
     }
-    if (nacc > 0 && w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
+    if (nacc > 0 && w < image_words) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
 }
 
 // Copy the image out with aligned dword stores (bytes at the two ragged ends).
@@ -563,19 +604,22 @@ __device__ __forceinline__ void kvc_front_k(const KvcStoreArgs &a, int64_t tile,
         g0 = g1 = kvc_stored_params(a, row);
     }
     const KvcPackedParams pp = kvc_packed_params(g0, g1);
-    if (act) {
-#pragma unroll 8
-        for (int t = 0; t < KVC_WAVE; t++) {
-            const uint32_t u = kvc_quant_pair_biased(*reinterpret_cast<const uint32_t *>(p + t * stride), pp);
-            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int nd = D >> 2;
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
+    for (int j = 0; j < 32; j++) v[j] = 0u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {                         // 32 tokens at a time through the staging area
+        if (act) {
+#pragma unroll 8
+            for (int t = 0; t < 32; t++) {
+                const uint32_t u = kvc_quant_pair_biased(*reinterpret_cast<const uint32_t *>(p + (32 * h + t) * stride), pp);
+                *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
+            }
+        }
+        kvc_wave_lds_sync();
+        kvc_read_k_rows(s_sym, RS, nd, lane, h, v);
+        kvc_wave_lds_sync();
+    }
 }
 
 // The count pass's variant: the lane keeps its two channels of all 64 tokens in registers (kvc_front_k_load: 64 loads in
@@ -626,19 +670,22 @@ __device__ __forceinline__ void kvc_front_k_once(const KvcStoreArgs &a, int64_t 
         g0 = g1 = kvc_stored_params(a, row);
     }
     const KvcPackedParams pp = kvc_packed_params(g0, g1);
-    if (act) {
-#pragma unroll
-        for (int t = 0; t < KVC_WAVE; t++) {
-            const uint32_t u = kvc_quant_pair_biased(raw[t], pp);
-            *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int nd = D >> 2;
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = j < nd ? *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j) : 0u;
+    for (int j = 0; j < 32; j++) v[j] = 0u;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {                         // 32 tokens at a time through the staging area
+        if (act) {
+#pragma unroll
+            for (int t = 0; t < 32; t++) {
+                const uint32_t u = kvc_quant_pair_biased(raw[32 * h + t], pp);
+                *reinterpret_cast<uint16_t *>(s_sym + t * RS + 2 * lane) = (uint16_t)kvc_low_bytes4(u, u);
+            }
+        }
+        kvc_wave_lds_sync();
+        kvc_read_k_rows(s_sym, RS, nd, lane, h, v);
+        kvc_wave_lds_sync();
+    }
 }
 
 // V tile: 128 tokens x 64 flat channels.  While the tile is quantized, lane l owns channels 2 (l & 31), + 1 of
@@ -662,7 +709,7 @@ __device__ __forceinline__ void kvc_front_v_load(const KvcStoreArgs &a, int64_t 
 __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile, int lane, uint8_t *s_sym, uint32_t *s_par,
                                             const uint32_t (&raw)[KVC_WAVE], uint32_t (&v)[32])
 {
-    constexpr int RS = KVC_V_TOKENS + 4;
+    constexpr int RS = 32 + 4;
     const int64_t row = tile / a.e.cols, col = tile - row * a.e.cols;
     const int pr = lane & 31, half = lane >> 5;
     const int64_t b = (col * KVC_WAVE) / ((int64_t)a.H * a.D);
@@ -674,30 +721,33 @@ __device__ __forceinline__ void kvc_front_v(const KvcStoreArgs &a, int64_t tile,
         const KvcPackedParams pp = kvc_packed_params(g, g);          // the token's constants in both halves
         *reinterpret_cast<uint4 *>(s_par + 4 * t) = make_uint4(pp.P2, pp.S2, pp.r2, pp.c2);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    kvc_wave_lds_sync();
 #pragma unroll
-    for (int jj = 0; jj < 16; jj++) {
-        uint32_t u[4];
+    for (int q = 0; q < 4; q++) {                         // a quarter of the tile at a time: tokens 16 q .. + 15 of either half
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int t = 64 * half + 4 * jj + k;
-            const uint4 c = *reinterpret_cast<const uint4 *>(s_par + 4 * t);
-            const KvcPackedParams pp = {c.x, c.y, c.z, c.w};
-            u[k] = kvc_quant_pair_biased(raw[4 * jj + k], pp);
+        for (int jj = 4 * q; jj < 4 * q + 4; jj++) {
+            uint32_t u[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                const int t = 64 * half + 4 * jj + k;
+                const uint4 c = *reinterpret_cast<const uint4 *>(s_par + 4 * t);
+                const KvcPackedParams pp = {c.x, c.y, c.z, c.w};
+                u[k] = kvc_quant_pair_biased(raw[4 * jj + k], pp);
+            }
+            // a01 = {channel 2 pr, 2 pr + 1 of token 4 jj | the same of token 4 jj + 1}; then four tokens of each channel
+            const uint32_t a01 = kvc_low_bytes4(u[0], u[1]), a23 = kvc_low_bytes4(u[2], u[3]);
+            const uint32_t w0 = kvc_low_bytes4(a01, a23), w1 = __builtin_amdgcn_perm(a23, a01, 0x07050301u);
+            *reinterpret_cast<uint32_t *>(s_sym + (2 * pr) * RS + 16 * half + 4 * (jj - 4 * q)) = w0;
+            *reinterpret_cast<uint32_t *>(s_sym + (2 * pr + 1) * RS + 16 * half + 4 * (jj - 4 * q)) = w1;
         }
-        // a01 = {channel 2 pr, 2 pr + 1 of token 4 jj | the same of token 4 jj + 1}; then four tokens of each channel
-        const uint32_t a01 = kvc_low_bytes4(u[0], u[1]), a23 = kvc_low_bytes4(u[2], u[3]);
-        const uint32_t w0 = kvc_low_bytes4(a01, a23), w1 = __builtin_amdgcn_perm(a23, a01, 0x07050301u);
-        *reinterpret_cast<uint32_t *>(s_sym + (2 * pr) * RS + 64 * half + 4 * jj) = w0;
-        *reinterpret_cast<uint32_t *>(s_sym + (2 * pr + 1) * RS + 64 * half + 4 * jj) = w1;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        kvc_wave_lds_sync();
 #pragma unroll
-    for (int j = 0; j < 32; j++) v[j] = *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * j);
+        for (int k = 0; k < 4; k++) {                     // register j holds tokens 4 j .. 4 j + 3 of the lane's channel
+            v[4 * q + k] = *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 4 * k);
+            v[16 + 4 * q + k] = *reinterpret_cast<const uint32_t *>(s_sym + lane * RS + 16 + 4 * k);
+        }
+        kvc_wave_lds_sync();                               // read: the area may take the next quarter
+    }
 }
 
 template <bool IS_K>
@@ -777,26 +827,34 @@ __global__ void __launch_bounds__(KVC_WG) kvc_store_emit_kernel(KvcStoreArgs a)
 // Two levels of status words.  A tile's is its own block_info, read and written as one 64-bit word
 // {u32 offset; u16 byte_num; u16 state}: a launch before this one marks every tile KVC_BI_NOT_READY, a wave that
 // knows its size writes {0, byte_num, KVC_BI_SIZE}, and once it knows its offset the final {offset, byte_num, 0}
-// (the reference's layout, state = padding = 0).  Runs of 64 consecutive tiles form a group with a word
+// (the reference's layout, state = padding = 0).  Runs of 56 consecutive tiles form a group with a word
 // {u32 bytes; u32 state} in the call's scratch slot: the wave of a group's last tile adds up the group
 // (KVC_BI_SIZE) and, once it knows what lies in front of the group, publishes the bytes up to the group's end
 // (state 0).  So a wave reads the sizes of the tiles before it in its own group (one 64-lane look), then walks the
 // group words backwards, 64 per look, adding sizes until a group with a known end stops the walk; tiles in flight
 // span a few dozen groups, so that is one or two looks.  Words that are not ready are polled again.
-// Progress: tiles are handed to workgroups in launch order, a wave publishes its size before it waits for anything,
-// and a group's size only needs the sizes of its own tiles, so whatever a wave waits for is published by waves that
-// started no later than itself and wait for nothing before publishing.  A wave that has polled KVC_LOOKBACK_POLLS
-// times gives up, flags the call (KVC_ENC_ERR_ORDER) and publishes what it has, so that every wave ends.
+//
+// Progress.  Two rules make every wait end: (1) a workgroup takes its tiles from a ticket counter when it starts
+// (not from its index in the launch, whose order of execution HIP does not promise), so every tile before a wave's
+// own belongs to a workgroup that has started; (2) a wave waits for nothing until the sizes of ALL its tiles are
+// published, and a group's size only needs the sizes of its own tiles.  So whatever a wave waits for is published
+// by waves that are running and wait for nothing before they publish.  (Placing a run's first tile before its
+// second was counted breaks rule 2 and turns the launch into one chain from wave to wave: 18 ms instead of 0.2.)
+// A wave that has found a word not ready more than max_polls times gives up all the same, flags the call
+// (KVC_ENC_ERR_ORDER) and publishes what it has, so that every wave ends; kvc_encode_finish_kernel then encodes the
+// whole call again the slow, safe way (two passes inside one workgroup), so a give-up costs time, not the result.
 constexpr uint32_t KVC_BI_SIZE = 1u, KVC_BI_NOT_READY = 0xffffu;
 constexpr uint32_t KVC_ENC_ERR_ORDER = 16u;         // a tile waited too long for the tiles before it
 constexpr uint32_t KVC_NO_CODE_LEN = 0x4000u;       // length of a symbol without a code: shows in any sum of lengths
-constexpr int KVC_LOOKBACK_POLLS = 1 << 18;         // some tenths of a second
 // The scratch slot of a one-pass call, in 32-bit words.  Tens of thousands of waves read the first tile's offset and
 // thousands of workgroups report maxima: on one cache line those accesses queue up behind each other (measured:
 // 0.5 ms of a 1.1 ms launch), so the offset gets a line that nothing is written to while the kernel runs, and the
 // maxima go to one of 32 lines picked by the workgroup number (kvc_encode_finish_kernel joins them afterwards).
+// The ticket counter shares the line of the call's status words, which nobody touches before the last tile is placed.
+constexpr int KVC_ONCE_POLLS_WORD = 6;               // status word: most looks of one wave that found a word not ready
+constexpr int KVC_ONCE_TICKET_WORD = 16;             // workgroups started so far
 constexpr int KVC_ONCE_BASE_WORD = 32;               // copy of status[KVC_ENC_ST_BASE]
-constexpr int KVC_ONCE_PART_WORD = 64, KVC_ONCE_PART_LINES = 32, KVC_ONCE_PART_STRIDE = 32;   // {error bits, largest tile, longest stream}
+constexpr int KVC_ONCE_PART_WORD = 64, KVC_ONCE_PART_LINES = 32, KVC_ONCE_PART_STRIDE = 32;   // {error bits, largest tile, longest stream, polls}
 constexpr int KVC_ONCE_GROUP_WORD = KVC_ONCE_PART_WORD + KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE;
 constexpr int KVC_ONCE_MAX_GROUPS = (int)((KVC_WS_SLOT_BYTES - KVC_ONCE_GROUP_WORD * 4) / 8);
 // Tiles per group: seven workgroups of a run-of-two launch, not eight.  Workgroups go to the chip's eight dies in turn,
@@ -837,32 +895,10 @@ __global__ void __launch_bounds__(KVC_WG) kvc_encode_mark_kernel(KvcEncodeArgs a
     if (tile < (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES) kvc_group_words(a)[tile] = kvc_group_word(0u, KVC_BI_NOT_READY);
     if (blockIdx.x == 0) {
         for (int i = threadIdx.x; i < KVC_ONCE_PART_LINES * KVC_ONCE_PART_STRIDE; i += KVC_WG) a.status[KVC_ONCE_PART_WORD + i] = 0u;
-        if (threadIdx.x == 0) a.status[KVC_ONCE_BASE_WORD] = a.status[KVC_ENC_ST_BASE];
-    }
-}
-
-// After the one-pass kernel: joins what the workgroups reported on their 32 lines into the call's status words.
-__global__ void __launch_bounds__(KVC_WAVE) kvc_encode_finish_kernel(KvcEncodeArgs a)
-{
-    const int lane = threadIdx.x;
-    uint32_t err = 0, tile = 0, stream = 0;
-    if (lane < KVC_ONCE_PART_LINES) {
-        const uint32_t *p = a.status + KVC_ONCE_PART_WORD + lane * KVC_ONCE_PART_STRIDE;
-        err = p[0];
-        tile = p[1];
-        stream = p[2];
-    }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        err |= (uint32_t)__shfl_xor((int)err, o, 64);
-        const uint32_t t = (uint32_t)__shfl_xor((int)tile, o, 64), st = (uint32_t)__shfl_xor((int)stream, o, 64);
-        tile = t > tile ? t : tile;
-        stream = st > stream ? st : stream;
-    }
-    if (lane == 0) {
-        a.status[1] |= err;
-        a.status[2] = tile;
-        a.status[3] = stream;
+        if (threadIdx.x == 0) {
+            a.status[KVC_ONCE_BASE_WORD] = a.status[KVC_ENC_ST_BASE];
+            a.status[KVC_ONCE_TICKET_WORD] = 0u;
+        }
     }
 }
 
@@ -899,7 +935,7 @@ __device__ __forceinline__ uint32_t kvc_look_back_in_group(const KvcEncodeArgs &
             in_group = kvc_wave_sum_u32(lane < r ? (uint32_t)(w >> 32) & 0xffffu : 0u);
             break;
         }
-        if (++*polls > KVC_LOOKBACK_POLLS) break;
+        if (++*polls > a.max_polls) break;
         __builtin_amdgcn_s_sleep(2);
         w = lane < r ? kvc_status_load(bi64 + group * KVC_ONCE_GROUP_TILES + lane) : 0ull;
     }
@@ -918,7 +954,7 @@ __device__ __forceinline__ uint32_t kvc_look_back_groups(const KvcEncodeArgs &a,
     uint32_t before = 0;
     int64_t j = group - 1;                                 // nearest group not yet accounted for
     uint64_t w = first_look;                               // taken at j = group - 1
-    while (j >= 0 && *polls <= KVC_LOOKBACK_POLLS) {
+    while (j >= 0 && *polls <= a.max_polls) {
         const uint32_t state = (uint32_t)(w >> 32), bytes = (uint32_t)w;
         const uint64_t not_ready = __ballot(state == KVC_BI_NOT_READY), known = __ballot(state == 0u);
         const int first_nr = not_ready ? __builtin_ctzll(not_ready) : 64, first_kn = known ? __builtin_ctzll(known) : 64;
@@ -954,11 +990,24 @@ __device__ __forceinline__ void kvc_load_code_table_marked(const KvcEncodeArgs &
     }
 }
 
-// A tile whose payload is packed (in the wave's second LDS area) but not yet placed; the words its look-back reads
-// were asked for when its size was published.
-// payloads up to this size wait in LDS; larger tiles are placed at once (a V tile has half the symbols of a K tile of
-// head_dim 128 and needs LDS for its tokens' constants)
-constexpr int kvc_once_keep_bytes(int front) { return front == 2 ? 2048 : 4096; }
+// LDS of one wave of the one-pass kernel: for V from fp16 the tokens' constants, then one area that holds the payload
+// images from its start upwards and the staging area of the tile front end at its top.  A payload of any size (at
+// most KVC_MAX_TILE_BYTES) leaves the staging area free, so a run's first tile can always wait in LDS while the second
+// is staged and counted; the second tile's image goes behind the first one's when both fit (it may then run into the
+// staging area, which is free by then), and otherwise the first tile is placed and written out before the second is
+// packed -- with both sizes published long before, so that nobody waits for this wave in the meantime.
+constexpr int KVC_ONCE_WAVE_BYTES = 12560;               // three workgroups of four waves per compute unit (160 KB)
+constexpr int kvc_once_par_bytes(int front) { return front == 2 ? 4 * KVC_V_TOKENS * 4 : 0; }
+constexpr int kvc_once_stage_bytes(int front) { return front == 1 ? KVC_STAGE_K_BYTES : front == 2 ? KVC_STAGE_VF16_BYTES : KVC_STAGE_VSYM_BYTES; }
+constexpr int kvc_once_area_bytes(int front) { return KVC_ONCE_WAVE_BYTES - kvc_once_par_bytes(front); }
+static_assert(KVC_STAGE_VSYM_BYTES >= KVC_STAGE_K_BYTES, "symbols in: the staging area serves K and V tiles");
+static_assert(kvc_once_area_bytes(0) - kvc_once_stage_bytes(0) >= KVC_IMAGE_WORDS * 4 &&
+              kvc_once_area_bytes(1) - kvc_once_stage_bytes(1) >= KVC_IMAGE_WORDS * 4 &&
+              kvc_once_area_bytes(2) - kvc_once_stage_bytes(2) >= KVC_IMAGE_WORDS * 4, "the largest payload must leave the staging area free");
+__device__ __forceinline__ uint32_t kvc_once_image_words(uint32_t bn) { return (bn + 3u) / 4u + 1u; }
+
+// A tile whose payload is packed but not yet placed; the words its look-back reads were asked for when its size was
+// published.
 struct KvcOncePending {
     int64_t tile;                                          // -1: nothing pending
     uint32_t bn, in_group;
@@ -987,7 +1036,7 @@ __device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const
     }
     *off_out = off;
     uint32_t err = 0;
-    const bool gave_up = *polls > KVC_LOOKBACK_POLLS;
+    const bool gave_up = *polls > a.max_polls;
     if (lane == 0) kvc_status_store(reinterpret_cast<uint64_t *>(a.block_infos) + tile, kvc_bi_word(off, bn, 0u));
     if (gave_up) err |= KVC_ENC_ERR_ORDER;
     KvcEmitPlace p;
@@ -1012,40 +1061,46 @@ __device__ __forceinline__ uint32_t kvc_once_place(const KvcEncodeArgs &a, const
 // A wave works through `run` (one or two) consecutive tiles.  For each it counts (symbols -> codes and lengths,
 // thread_infos), publishes the size, asks for the words its look-back will read and packs the payload into LDS as an
 // image that starts on a word (where the payload goes is not needed for that).  The first tile of a run of two stays in
-// the wave's second LDS area until the second is packed too; then one look-back finds the first tile's place, the second
+// LDS until the second is counted and packed too; then one look-back finds the first tile's place, the second
 // follows right behind it, and both are written out.  So a tile is placed a whole tile's work after its size was
 // published, when the tiles before it have published theirs: with the look-back right behind the count, a tile waits
 // 10 us on average for the slowest of the thousands of tiles in flight before it (measured), as long as the rest of
 // its work takes.
 // Dynamic LDS: the encode table (one for the workgroup, or one per wave when tile rows have codebooks of their own:
-// then run = 1), then per wave the tile of symbols, for V the tokens' constants, and the kept payload image.
+// then run = 1), then KVC_ONCE_WAVE_BYTES per wave.
 template <int FRONT>
 __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs a, int run)
 {
     extern __shared__ __align__(16) uint8_t s_dyn[];
-    __shared__ uint32_t s_short[KVC_WAVES_PER_WG], s_err, s_max_tile, s_longest;
+    __shared__ uint32_t s_short[KVC_WAVES_PER_WG], s_err, s_max_tile, s_longest, s_polls, s_ticket;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const bool own_table = a.e.rows_per_codebook != 0;
     uint2 *s_table = reinterpret_cast<uint2 *>(s_dyn) + (own_table ? wave * 256 : 0);
-    uint8_t *per_wave = s_dyn + (own_table ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2);
-    constexpr int PAR_BYTES = FRONT == 2 ? 4 * KVC_V_TOKENS * 4 : 0;
-    constexpr int KEEP_BYTES = kvc_once_keep_bytes(FRONT);
-    uint8_t *s_sym = per_wave + wave * (KVC_SYM_TILE_BYTES + PAR_BYTES + KEEP_BYTES + 16);
-    uint32_t *s_par = reinterpret_cast<uint32_t *>(s_sym + KVC_SYM_TILE_BYTES);
-    uint32_t *kept = reinterpret_cast<uint32_t *>(s_sym + KVC_SYM_TILE_BYTES + PAR_BYTES);
-    const int64_t tile0 = ((int64_t)blockIdx.x * KVC_WAVES_PER_WG + wave) * run;
+    uint8_t *s_wave = s_dyn + (own_table ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2) + wave * KVC_ONCE_WAVE_BYTES;
+    constexpr int PAR_BYTES = kvc_once_par_bytes(FRONT), AREA_BYTES = kvc_once_area_bytes(FRONT);
+    uint32_t *s_par = reinterpret_cast<uint32_t *>(s_wave);
+    uint32_t *area = reinterpret_cast<uint32_t *>(s_wave + PAR_BYTES);
+    uint8_t *s_stage = s_wave + PAR_BYTES + AREA_BYTES - kvc_once_stage_bytes(FRONT);
     uint32_t *my_short = &s_short[own_table ? wave : 0];
-    if (tid == 0) { s_err = 0; s_max_tile = 0; s_longest = 0; }
+    // the workgroup's ticket: which tiles it takes (the table of a call with one codebook is fetched meanwhile)
+    uint32_t ticket = 0;
+    if (tid == 0) ticket = atomicAdd(&a.e.status[KVC_ONCE_TICKET_WORD], 1u);
     if (lane == 0) s_short[wave] = 1u;
+    if (!own_table && wave == 0) kvc_load_code_table_marked(a.e, 0, s_table, my_short, lane);
+    if (tid == 0) { s_err = 0; s_max_tile = 0; s_longest = 0; s_polls = 0; s_ticket = ticket; }
     __syncthreads();
-    if (own_table ? tile0 < a.e.tiles : wave == 0) kvc_load_code_table_marked(a.e, tile0 < a.e.tiles ? tile0 : 0, s_table, my_short, lane);
-    __syncthreads();
+    const int64_t tile0 = ((int64_t)s_ticket * KVC_WAVES_PER_WG + wave) * run;
+    if (own_table) {
+        if (tile0 < a.e.tiles) kvc_load_code_table_marked(a.e, tile0, s_table, my_short, lane);
+        __syncthreads();
+    }
     const bool short_codes = *my_short != 0u;              // wave-uniform
     const int nd = a.e.vec_len >> 2;
     uint64_t *bi64 = reinterpret_cast<uint64_t *>(a.e.block_infos);
     const uint32_t base = a.e.status[KVC_ONCE_BASE_WORD];
-    uint32_t err = 0, max_tile = 0, longest = 0;
+    uint32_t err = 0, max_tile = 0, longest = 0, next_off = 0;
     int polls = 0;
+    bool first_placed = false;
     KvcOncePending pd;
     pd.tile = -1;
     uint32_t raw[KVC_WAVE];                                // a tile as loaded from fp16: two channels of 64 tokens per lane
@@ -1053,21 +1108,25 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
     for (int it = 0; it < run; it++) {
         const int64_t tile = tile0 + it;
         if (tile >= a.e.tiles) break;
+        // (the lane number made opaque: what the front ends derive from it -- some dozens of LDS and global addresses --
+        // is then worked out where it is used instead of being kept in registers across the whole loop body)
+        int lane = tid & 63;
+        asm volatile("" : "+v"(lane));
         uint32_t v[32];
         if constexpr (FRONT == 1) {
             // the loads of the run's second tile are on their way while the first is counted and packed
             if (it == 0) kvc_front_k_load(a, tile, lane, raw);
-            kvc_front_k_once(a, tile, lane, s_sym, raw, v);
+            kvc_front_k_once(a, tile, lane, s_stage, raw, v);
             if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_k_load(a, tile + 1, lane, raw);
         } else if constexpr (FRONT == 2) {
             if (it == 0) kvc_front_v_load(a, tile, lane, raw);
-            kvc_front_v(a, tile, lane, s_sym, s_par, raw, v);
+            kvc_front_v(a, tile, lane, s_stage, s_par, raw, v);
             if (it + 1 < run && tile + 1 < a.e.tiles) kvc_front_v_load(a, tile + 1, lane, raw);
         } else {
-            if (a.e.is_k) kvc_load_vector_k_tile(a.e, tile, lane, s_sym, v);
-            else kvc_load_vector_v_tile(a.e, tile, lane, s_sym, v);       // (the launcher requires 4-byte aligned symbols and rows)
+            if (a.e.is_k) kvc_load_vector_k_tile(a.e, tile, lane, s_stage, v);
+            else kvc_load_vector_v_tile(a.e, tile, lane, s_stage, v);       // (the launcher requires 4-byte aligned symbols and rows)
         }
-        kvc_wave_lds_sync();                               // every lane holds its vector: the tile area is free
+        // (every lane holds its vector and the staging area is free: the front ends finish with a hand-over)
         uint32_t bits = 0;
         uint32_t gl[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u}; // short codes: the four group lengths of registers 4 i .. 4 i + 3
         if (short_codes) {
@@ -1117,11 +1176,26 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
         if (pd.tile < 0 || cur.in_group_known) cur.looks = kvc_look_back_ask(a.e, tile, lane);    // (a tile that follows a kept one looks at nothing)
         if (cur.in_group_known) cur.in_group = kvc_look_back_in_group(a.e, tile, bn, lane, cur.looks.tile_word, &polls);
         cur.packs = bn <= (uint32_t)KVC_MAX_TILE_BYTES;
-        const bool keep = bn <= (uint32_t)KEEP_BYTES && it + 1 < run && tile + 1 < a.e.tiles;
-        uint32_t *image = keep ? kept : reinterpret_cast<uint32_t *>(s_sym);
+        // where this tile's image goes: behind the kept one's, or -- the two do not fit the area together (more than six
+        // bits per symbol on average) -- to the start of the area once the kept tile has been placed and written out.
+        // The sizes of both tiles are published by now: this wave's wait holds nobody up.
+        const uint32_t my_words = kvc_once_image_words(bn);
+        uint32_t *image = area;
+        if (pd.tile >= 0) {
+            const uint32_t kept_words = pd.packs ? kvc_once_image_words(pd.bn) : 0u;
+            if (cur.packs && (kept_words + my_words) * 4u > (uint32_t)AREA_BYTES) {
+                uint32_t off = 0;
+                err |= kvc_once_place(a.e, pd, area, base, lane, &polls, &off);
+                next_off = off + pd.bn;
+                first_placed = true;
+                pd.tile = -1;
+                kvc_wave_lds_sync();                       // the kept image is read: the area is free
+            } else {
+                image = area + kept_words;
+            }
+        }
         if (cur.packs) {
-            const uint32_t image_words = (bn + 3u) / 4u + 1u;
-            for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
+            for (uint32_t i = lane; i < my_words; i += KVC_WAVE) image[i] = 0;
             kvc_wave_lds_sync();
             if (short_codes) {
                 const uint32_t bitpos = start * 8u;
@@ -1136,43 +1210,179 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
                             nacc += len;
                             if (nacc >= 32u) {
                                 nacc -= 32u;
-                                if (w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
+                                if (w < my_words) atomicOr(&image[w], kvc_bswap((uint32_t)(acc >> nacc)));
                                 w++;
                             }
                         }
                     }
-                    if (nacc > 0 && w < (uint32_t)KVC_IMAGE_WORDS) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
+                    if (nacc > 0 && w < my_words) atomicOr(&image[w], kvc_bswap((uint32_t)(acc << (32u - nacc))));
                 }
             } else if (!bad) {
-                kvc_pack_vector(a.e, start, v, s_table, image, 0u, false);
+                kvc_pack_vector(a.e, start, v, s_table, image, 0u, false, my_words);
             }
             kvc_wave_lds_sync();
         }
-        if (keep) {
+        if (it + 1 < run && tile + 1 < a.e.tiles) {
             pd = cur;                                      // placed together with the next tile
             continue;
         }
         uint32_t off = 0;
         if (pd.tile >= 0) {                                // the kept tile, whose words have had this tile's work to arrive
-            err |= kvc_once_place(a.e, pd, kept, base, lane, &polls, &off);
+            err |= kvc_once_place(a.e, pd, area, base, lane, &polls, &off);
             err |= kvc_once_place(a.e, cur, image, base, lane, &polls, &off, true, off + pd.bn);
             pd.tile = -1;
-        } else {                                           // a run of one, or the tile before was too large to keep
+        } else if (first_placed) {                         // the kept tile went out before this one was packed
+            err |= kvc_once_place(a.e, cur, image, base, lane, &polls, &off, true, next_off);
+        } else {                                           // a run of one
             err |= kvc_once_place(a.e, cur, image, base, lane, &polls, &off);
         }
-        kvc_wave_lds_sync();                               // the images are read: the areas may take the next tiles
     }
     if (lane == 0 && tile0 < a.e.tiles) {
         if (err) atomicOr(&s_err, err);
         atomicMax(&s_max_tile, max_tile);
         atomicMax(&s_longest, longest);
+        atomicMax(&s_polls, (uint32_t)polls);
     }
     __syncthreads();
-    if (tid == 0) {                                        // to this workgroup's line of the slot
-        uint32_t *part = a.e.status + KVC_ONCE_PART_WORD + (blockIdx.x % KVC_ONCE_PART_LINES) * KVC_ONCE_PART_STRIDE;
+    if (tid == 0) {                                        // to one of the slot's lines, picked by the ticket
+        uint32_t *part = a.e.status + KVC_ONCE_PART_WORD + (s_ticket % KVC_ONCE_PART_LINES) * KVC_ONCE_PART_STRIDE;
         if (s_err) atomicOr(&part[0], s_err);
         atomicMax(&part[1], s_max_tile);
         atomicMax(&part[2], s_longest);
+        atomicMax(&part[3], s_polls);
+    }
+}
+
+// After the one-pass kernel, one workgroup: joins what the workgroups reported on their 32 lines into the call's status
+// words.  If a wave gave up on its look-back (KVC_ENC_ERR_ORDER: the payload and the block_infos are then incomplete)
+// this workgroup encodes the whole call again in two passes of its own -- count every tile, add up the offsets, emit
+// every tile: nothing in it waits for another workgroup, so it always ends, and since the inputs are untouched the
+// outputs are the ones the call was to produce.  Slow (four waves for all tiles), and next to never needed: the
+// look-back's progress does not depend on the order in which the hardware starts workgroups.
+template <int FRONT>
+__global__ void __launch_bounds__(KVC_WG) kvc_encode_finish_kernel(KvcStoreArgs a)
+{
+    __shared__ uint2 s_table[KVC_WAVES_PER_WG][256];
+    __shared__ uint8_t s_len[KVC_WAVES_PER_WG][256];
+    __shared__ __align__(16) uint8_t s_sym[KVC_WAVES_PER_WG][KVC_SYM_TILE_BYTES];   // staging area first, then the payload image
+    __shared__ __align__(16) uint32_t s_par[FRONT == 2 ? KVC_WAVES_PER_WG : 1][FRONT == 2 ? 4 * KVC_V_TOKENS : 4];
+    __shared__ uint32_t s_short[KVC_WAVES_PER_WG], s_err, s_longest, s_again;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    if (wave == 0) {
+        uint32_t err = 0, tile = 0, stream = 0, polls = 0;
+        if (lane < KVC_ONCE_PART_LINES) {
+            const uint32_t *p = a.e.status + KVC_ONCE_PART_WORD + lane * KVC_ONCE_PART_STRIDE;
+            err = p[0];
+            tile = p[1];
+            stream = p[2];
+            polls = p[3];
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            err |= (uint32_t)__shfl_xor((int)err, o, 64);
+            const uint32_t t = (uint32_t)__shfl_xor((int)tile, o, 64), st = (uint32_t)__shfl_xor((int)stream, o, 64);
+            const uint32_t po = (uint32_t)__shfl_xor((int)polls, o, 64);
+            tile = t > tile ? t : tile;
+            stream = st > stream ? st : stream;
+            polls = po > polls ? po : polls;
+        }
+        if (a.e.force_order) err |= KVC_ENC_ERR_ORDER;
+        if (lane == 0) {
+            a.e.status[KVC_ONCE_POLLS_WORD] = polls;
+            s_again = err & KVC_ENC_ERR_ORDER;
+            if (!(err & KVC_ENC_ERR_ORDER)) {
+                a.e.status[1] |= err;
+                a.e.status[2] = tile;
+                a.e.status[3] = stream;
+            }
+            s_err = 0;
+            s_longest = 0;
+        }
+    }
+    __syncthreads();
+    if (!s_again) return;
+    // ---- the whole call again, two passes inside this workgroup ----
+    const int64_t tiles = a.e.tiles;
+    for (int64_t tile = wave; tile < tiles; tile += KVC_WAVES_PER_WG) {      // count: thread_infos, byte_nums, group parameters
+        kvc_load_len_table(a.e, tile, s_len[wave], lane);
+        kvc_wave_lds_sync();
+        uint32_t v[32];
+        if constexpr (FRONT == 1) {
+            uint32_t raw[KVC_WAVE];
+            kvc_front_k_load(a, tile, lane, raw);
+            kvc_front_k_once(a, tile, lane, s_sym[wave], raw, v);
+        } else if constexpr (FRONT == 2) {
+            uint32_t raw[KVC_WAVE];
+            kvc_front_v_load(a, tile, lane, raw);
+            kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], raw, v);
+        } else {
+            kvc_load_vector(a.e, tile, lane, v);
+        }
+        const uint32_t longest = kvc_count_tile(a.e, tile, lane, v, s_len[wave], &s_err);
+        if (lane == 0) atomicMax(&s_longest, longest);
+        kvc_wave_lds_sync();
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (wave == 0) {                                                         // offsets, in tile order
+        uint32_t *bi = reinterpret_cast<uint32_t *>(a.e.block_infos);
+        const uint32_t base = a.e.status[KVC_ENC_ST_BASE];
+        uint32_t at = base, largest = 0;
+        for (int64_t t0 = 0; t0 < tiles; t0 += KVC_WAVE) {
+            const int64_t tile = t0 + lane;
+            const uint32_t bn = tile < tiles ? bi[2 * tile + 1] & 0xffffu : 0u;
+            const uint32_t incl = kvc_wave_inclusive_scan(bn, lane);
+            if (tile < tiles) bi[2 * tile] = at + incl - bn;
+            at += (uint32_t)__builtin_amdgcn_readlane((int)incl, KVC_WAVE - 1);
+            const uint32_t m = kvc_wave_max_dpp(bn);
+            largest = m > largest ? m : largest;
+        }
+        if (lane == 0) {
+            const uint32_t total = at - base;
+            a.e.status[0] = total;
+            a.e.status[2] = largest;
+            if ((int64_t)(base - a.e.base_global_offset) + total > a.e.encoded_cap) atomicOr(&s_err, KVC_ENC_ERR_CAPACITY);
+            if (a.e.idx_offset) {
+                a.e.idx_offset[0] = (uint32_t)tiles;
+                a.e.idx_offset[1] = total;
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    for (int64_t tile = wave; tile < tiles; tile += KVC_WAVES_PER_WG) {      // emit
+        if (lane == 0) s_short[wave] = 1u;
+        kvc_wave_lds_sync();
+        kvc_load_code_table(a.e, tile, s_table[wave], &s_short[wave], lane);
+        kvc_wave_lds_sync();
+        const KvcEmitPlace p = kvc_emit_place(a.e, tile, true);
+        if (!p.ok) continue;                                                 // flagged by the count pass or the offsets
+        uint32_t *image = reinterpret_cast<uint32_t *>(s_sym[wave]);
+        uint32_t v[32];
+        if constexpr (FRONT == 1) {
+            kvc_front_k(a, tile, lane, s_sym[wave], v);
+        } else if constexpr (FRONT == 2) {
+            uint32_t raw[KVC_WAVE];
+            kvc_front_v_load(a, tile, lane, raw);
+            kvc_front_v(a, tile, lane, s_sym[wave], s_par[wave], raw, v);
+        } else {
+            kvc_load_vector(a.e, tile, lane, v);
+        }
+        kvc_wave_lds_sync();
+        const uint32_t image_words = (p.head + p.bn + 3u) / 4u + 1u;
+        for (uint32_t i = lane; i < image_words && i < (uint32_t)KVC_IMAGE_WORDS; i += KVC_WAVE) image[i] = 0;
+        kvc_wave_lds_sync();
+        kvc_pack_vector(a.e, kvc_stream_start(a.e, tile, lane), v, s_table[wave], image, p.head, s_short[wave] != 0u);
+        kvc_wave_lds_sync();
+        kvc_write_image(a.e, p, lane, image);
+        kvc_wave_lds_sync();
+    }
+    __syncthreads();
+    if (tid == 0) {
+        a.e.status[1] = (a.e.status[1] & KVC_ENC_ERR_CODEBOOK) | s_err;
+        a.e.status[3] = s_longest;
     }
 }
 
@@ -1256,6 +1466,8 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     a.idx_offset = reinterpret_cast<uint32_t *>(c.d_idx_offset);
     a.stream_bytes = c.d_stream_bytes;
     a.result = c.d_result;
+    a.max_polls = 0;
+    a.force_order = 0;
     const int64_t chunks = (a.tiles + 1023) / 1024;
     KVC_REQUIRE((KVC_ENC_STATUS_WORDS + chunks) * 4 <= (int64_t)KVC_WS_SLOT_BYTES, "too many tiles (%lld) for one encode call",
                 (long long)a.tiles);
@@ -1284,23 +1496,33 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     const bool symbols_in_one_pass = one_pass > 1 || (one_pass == 1 && a.tiles >= 8192);
     if ((src ? one_pass != 0 : symbols_in_one_pass) && ((uintptr_t)c.d_block_infos & 7) == 0 &&
         (a.tiles + KVC_ONCE_GROUP_TILES - 1) / KVC_ONCE_GROUP_TILES <= KVC_ONCE_MAX_GROUPS) {
-        if (!src) sa.e = a;
+        // how often a wave may find a word of its look-back not ready; -1 makes the call take the give-up path
+        // (every wave still ends normally) so that tests can reach it from the host
+        const int polls_opt = kvc_option(KVC_OPT_ENCODE_LOOKBACK_POLLS);
+        a.max_polls = polls_opt < 0 ? 0 : polls_opt;
+        a.force_order = polls_opt < 0;
+        sa.e = a;
         const int front = !src ? 0 : is_k ? 1 : 2;
-        const size_t lds = (size_t)(a.rows_per_codebook ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2) +
-                           (size_t)KVC_WAVES_PER_WG * (KVC_SYM_TILE_BYTES + (front == 2 ? 4 * KVC_V_TOKENS * 4 : 0) + kvc_once_keep_bytes(front) + 16);
+        const size_t lds = (size_t)(a.rows_per_codebook ? KVC_WAVES_PER_WG : 1) * 256 * sizeof(uint2) + (size_t)KVC_WAVES_PER_WG * KVC_ONCE_WAVE_BYTES;
         hipLaunchKernelGGL(kvc_encode_mark_kernel, dim3((unsigned)((a.tiles + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a);
         // two tiles per wave (the look-back of the first hides behind the count of the second) where all tiles share
-        // the codebook and there are enough of them to keep the chip full.  Longer runs would chain the groups: a wave
-        // would place a tile (which needs the sizes of all groups before it) before it counts and publishes a later one.
+        // the codebook and there are enough of them to keep the chip full.  Longer runs would need the payloads of
+        // more than one waiting tile in LDS.
         const int want = one_pass;
         int run = want == 1 ? (a.tiles >= 8192 ? 2 : 1) : want - 1;       // 2, 3: always one, two tiles per wave
         run = run < 1 ? 1 : run > 2 ? 2 : run;
         if (a.rows_per_codebook != 0) run = 1;
         const unsigned wgs1 = (unsigned)((a.tiles + (int64_t)run * KVC_WAVES_PER_WG - 1) / ((int64_t)run * KVC_WAVES_PER_WG));
-        if (front == 0) hipLaunchKernelGGL(kvc_encode_once_kernel<0>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
-        else if (front == 1) hipLaunchKernelGGL(kvc_encode_once_kernel<1>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
-        else hipLaunchKernelGGL(kvc_encode_once_kernel<2>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
-        hipLaunchKernelGGL(kvc_encode_finish_kernel, dim3(1), dim3(KVC_WAVE), 0, stream, a);
+        if (front == 0) {
+            hipLaunchKernelGGL(kvc_encode_once_kernel<0>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+            hipLaunchKernelGGL(kvc_encode_finish_kernel<0>, dim3(1), dim3(KVC_WG), 0, stream, sa);
+        } else if (front == 1) {
+            hipLaunchKernelGGL(kvc_encode_once_kernel<1>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+            hipLaunchKernelGGL(kvc_encode_finish_kernel<1>, dim3(1), dim3(KVC_WG), 0, stream, sa);
+        } else {
+            hipLaunchKernelGGL(kvc_encode_once_kernel<2>, dim3(wgs1), dim3(KVC_WG), lds, stream, sa, run);
+            hipLaunchKernelGGL(kvc_encode_finish_kernel<2>, dim3(1), dim3(KVC_WG), 0, stream, sa);
+        }
         if (a.result || a.stream_bytes) hipLaunchKernelGGL(kvc_encode_publish_kernel, dim3(1), dim3(1), 0, stream, a);
         KVC_HIP(hipGetLastError());
         *slot_out = slot;
