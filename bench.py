@@ -137,7 +137,7 @@ def cpu_baseline(kctx, q, k_fp16, cfg, budget_s=10.0):
     bits = O.py_bits(syms, book)
     dt = time.perf_counter() - t0
     legs["python_heapq_huffman"] = {"value": round(syms.size / dt / 1e9, 6), "unit": "GB/s symbols in", "cores": 1,
-                                    "sample": "65536 symbols of K, %d bits out, %.2f s (pure Python: not extrapolated)" % (bits.size, dt)}
+                                    "sample": "65536 symbols of K, %d bits out, %.1f ms (pure Python: not extrapolated)" % (bits.size, dt * 1e3)}
     out["legs"] = legs
     return out
 
@@ -310,6 +310,7 @@ def quick_attention(name, steps=50, warmup=10):
     kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
     kctx.store(k, want_symbols=False)
     vctx.store(v, want_symbols=False)
+    rates = codec_rates(kctx, vctx, k, v, cfg)           # encode / decode rates of the same prompt cache (GB/s)
     del k, v
     g = torch.Generator().manual_seed(1236)
     q = torch.randn(B, Hq, D, generator=g, dtype=torch.float32).to(torch.float16).to(dev)
@@ -338,13 +339,36 @@ def quick_attention(name, steps=50, warmup=10):
         attns[i % n].attend(q, out=out, kernel_ms=kms)
         k_ms += kms[0] / steps
         v_ms += kms[1] / steps
+    # the same step captured once in a HIP graph and replayed (where the step is launch-bound, this is what counts)
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        attns[0].attend(q, out=out)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            attns[0].attend(q, out=out)
+    torch.cuda.synchronize()
+    eager = attns[0].attend(q).clone()
+    for _ in range(warmup):
+        graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    graph_ms = (time.perf_counter() - t0) / steps * 1e3
+    assert torch.equal(out, eager), "%s: graph replay differs from the eager call" % name
+    del graph
     res = {"workload": cfg["desc"], "ms_per_step": round(ms, 4), "GBs": round((kb + vb) / (ms * 1e-3) / 1e9, 1),
            "pct_hbm_peak": round(100 * (kb + vb) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 2),
+           "graph_replay_ms_per_step": round(graph_ms, 4), "codec": rates,
            "kernels_ms": {"fused_k": round(k_ms, 4), "fused_v": round(v_ms, 4)}, "compressed_bytes": {"k": kb, "v": vb},
            "compression_ratio": {"k": round(kctx.get_cr(), 3), "v": round(vctx.get_cr(), 3)},
            "k_max_code_bits": kctx.max_code_bits, "v_max_code_bits": vctx.max_code_bits,
            "cache_copies_cycled": n, "steps": steps, "check_max_error": err}
-    log("[bench] %s: step %.3f ms (%.0f GB/s of compressed bytes), fused K %.3f ms, fused V %.3f ms" % (name, ms, res["GBs"], k_ms, v_ms))
+    log("[bench] %s: step %.3f ms (%.0f GB/s of compressed bytes; as a replayed graph %.3f ms), fused K %.3f ms, fused V %.3f ms; "
+        "fused store K %.0f / V %.0f GB/s of fp16 in" % (name, ms, res["GBs"], graph_ms, k_ms, v_ms,
+                                                        rates["k"]["store_fused_GBs_fp16_in"] or 0, rates["v"]["store_fused_GBs_fp16_in"] or 0))
     del attns, kctx, vctx
     torch.cuda.empty_cache()
     return res

@@ -109,6 +109,8 @@ class CompressedAttention:
 
     def _desc(self, ctx: KVCompCtx, lut) -> "_lib.CompressedDesc":
         d = _lib.CompressedDesc()
+        if ctx._probe is not None:
+            ctx.poll_stores()                              # what queued stores have left, if it has arrived: no wait
         if ctx.compressed_ctx_len:
             d.d_luts = lut.data_ptr()
             # (addresses and sizes straight from the contexts' growing arrays: a tensor view per field and call costs more

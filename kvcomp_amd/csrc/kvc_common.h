@@ -64,7 +64,7 @@ int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the
 // reference-signature entry points derive from the decode tree on every call.
 constexpr size_t KVC_WS_SLOT_BYTES = 16384;
-int kvc_workspace_slot(void **slot);
+int kvc_workspace_slot(void **slot, void *stream);   // stream: the one the call launches on (a recorded call gets a slot of its own)
 int kvc_quant_params(const void *d_x_f16, int64_t NB, int64_t BS, int64_t B, int64_t H, int64_t D, int quant_mask,
                      float eb, int8_t *d_min_i8, void *d_scale_f16, void *stream);
 int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_tree_bytes, int tree_format,

@@ -185,7 +185,7 @@ static int kvc_entropy_decode(int is_k, const uint8_t *d_encoded, int64_t encode
         if (rc != 1) return rc;
     }
     void *slot;
-    if (int rc = kvc_workspace_slot(&slot)) return rc;
+    if (int rc = kvc_workspace_slot(&slot, (void *)stream_)) return rc;
     KvcStreamArgs s;
     int64_t rows;
     if (int rc = kvc_fill_stream_args(s, d_encoded, encoded_bytes, d_block_infos, block_infos_bytes, d_thread_infos,

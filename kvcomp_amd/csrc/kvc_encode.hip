@@ -1442,7 +1442,7 @@ static int kvc_encode_launch(const KvcEncodeCall &c, void **slot_out, hipStream_
     KVC_REQUIRE(c.rows_per_codebook >= 0 && (c.rows_per_codebook == 0 || (c.table_stride >= c.table_bytes && c.table_stride % 8 == 0)),
                 "tables of several codebooks must be a multiple of 8 bytes apart and not overlap");
     void *slot;
-    if (int rc = kvc_workspace_slot(&slot)) return rc;
+    if (int rc = kvc_workspace_slot(&slot, (void *)stream)) return rc;
     KvcEncodeArgs a;
     a.sym = c.d_sym;
     a.stride = c.stride;

@@ -1000,7 +1000,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                 "quant_scales must be 4-byte aligned and quant_min_ints 2-byte aligned");
     void *slot = nullptr;
     if (!d_luts) {
-        if (int rc = kvc_workspace_slot(&slot)) return rc;
+        if (int rc = kvc_workspace_slot(&slot, stream_)) return rc;
     }
     KvcFusedArgs a;
     int64_t rows;
@@ -1093,7 +1093,7 @@ int kvc_expand(int is_k, int deq, const uint8_t *d_decode_tree, int64_t decode_t
     KVC_REQUIRE(!deq || (((uintptr_t)d_scale & 3) == 0 && ((uintptr_t)d_min & 1) == 0),
                 "quant_scales must be 4-byte aligned and quant_min_ints 2-byte aligned");
     void *slot = nullptr;
-    if (int rc = kvc_workspace_slot(&slot)) return rc;
+    if (int rc = kvc_workspace_slot(&slot, stream_)) return rc;
     KvcFusedArgs a;
     a.sched_nseg = 0;
     int64_t rows;

@@ -107,22 +107,42 @@ extern "C" int kvc_get_option(const char *name, int *value)
 // per-device scratch ring: KVC_WS_SLOTS slots handed out round-robin.  A slot is reused after
 // KVC_WS_SLOTS further calls, so at most that many calls may be in flight on different streams of one
 // device at the same time (calls on one stream are ordered anyway).
+// A call that is being recorded into a HIP graph runs again on every replay, long after the ring has come
+// round: it gets a slot of a second pool whose slots are handed out once and never again (at most
+// KVC_WS_CAPTURE_SLOTS recorded calls per device and process).  Both pools are allocated by the first call on
+// a device, which therefore must not be a recorded one.
 // ---------------------------------------------------------------------------------------------------
 constexpr int KVC_WS_SLOTS = 32;
+constexpr int KVC_WS_CAPTURE_SLOTS = 480;
 constexpr int KVC_MAX_DEVICES = 16;
 static std::mutex g_ws_mutex;
 static void *g_ws_base[KVC_MAX_DEVICES] = {};
 static unsigned g_ws_next[KVC_MAX_DEVICES] = {};
+static unsigned g_ws_captured[KVC_MAX_DEVICES] = {};
 
-int kvc_workspace_slot(void **slot)
+int kvc_workspace_slot(void **slot, void *stream)
 {
     int dev = 0;
     KVC_HIP(hipGetDevice(&dev));
     KVC_REQUIRE(dev >= 0 && dev < KVC_MAX_DEVICES, "device index %d out of range", dev);
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (stream) KVC_HIP(hipStreamIsCapturing((hipStream_t)stream, &capturing));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
-    if (!g_ws_base[dev]) KVC_HIP(hipMalloc(&g_ws_base[dev], KVC_WS_SLOTS * KVC_WS_SLOT_BYTES));
-    unsigned k = g_ws_next[dev]++ % KVC_WS_SLOTS;
-    *slot = (char *)g_ws_base[dev] + k * KVC_WS_SLOT_BYTES;
+    if (!g_ws_base[dev]) {
+        KVC_REQUIRE(capturing == hipStreamCaptureStatusNone,
+                    "the first call on a device allocates the library's scratch memory and cannot be recorded into a graph: "
+                    "make one call outside the capture first");
+        KVC_HIP(hipMalloc(&g_ws_base[dev], (size_t)(KVC_WS_SLOTS + KVC_WS_CAPTURE_SLOTS) * KVC_WS_SLOT_BYTES));
+    }
+    unsigned k;
+    if (capturing != hipStreamCaptureStatusNone) {
+        KVC_REQUIRE(g_ws_captured[dev] < (unsigned)KVC_WS_CAPTURE_SLOTS,
+                    "more than %d calls that need scratch memory have been recorded into graphs on this device", KVC_WS_CAPTURE_SLOTS);
+        k = KVC_WS_SLOTS + g_ws_captured[dev]++;
+    } else {
+        k = g_ws_next[dev]++ % KVC_WS_SLOTS;
+    }
+    *slot = (char *)g_ws_base[dev] + (size_t)k * KVC_WS_SLOT_BYTES;
     return 0;
 }
 

@@ -460,7 +460,7 @@ static int kvc_quant_launch(const void *d_x_f16, int64_t NB, int64_t BS, int64_t
         const int64_t groups = quant_mask == KVC_MASK_K_BLOCK ? NB : NB * B;
         KVC_REQUIRE(groups * 8 <= (int64_t)KVC_WS_SLOT_BYTES, "too many block-quantization groups (%lld) for one call", (long long)groups);
         void *slot;
-        if (int rc = kvc_workspace_slot(&slot)) return rc;
+        if (int rc = kvc_workspace_slot(&slot, (void *)stream)) return rc;
         a.minmax = reinterpret_cast<uint32_t *>(slot);
         const unsigned row_wgs = (unsigned)((rows + KVC_WAVES_PER_WG - 1) / KVC_WAVES_PER_WG);
         hipLaunchKernelGGL(kvc_quant_block_init_kernel, dim3((unsigned)((groups + KVC_WG - 1) / KVC_WG)), dim3(KVC_WG), 0, stream, a.minmax, groups);

@@ -211,6 +211,17 @@ class KVCompCtx:
         # word 8 counts the payload bytes in _encoded; _enc_pending bounds the bytes the host has not learnt of yet
         self._state: Optional[torch.Tensor] = None
         self._enc_pending = 0
+        # Stores that were queued and not yet seen to succeed, oldest first: (tokens, their fp16 rows or None, the
+        # bookkeeping as it stood right after the store, the store's share of _enc_pending, whether the tokens are gone
+        # if the store has to be taken back: counted in ctx_len, rows not kept); _verified is the
+        # bookkeeping behind the last store that is known to be good.  _probe = (event, stores covered) while a copy of
+        # the device words to _host_words (pinned) is on its way: reading it later costs no wait.
+        self._unverified: list = []
+        self._verified = None
+        self._probe = None
+        self._host_words: Optional[torch.Tensor] = None
+        self._trim_after_sync = False
+        self.waits = 0                     # how often this context has waited for the device to learn sizes
 
     def _device_state(self) -> torch.Tensor:
         if self._state is None:
@@ -218,16 +229,86 @@ class KVCompCtx:
             self._state[8] = self._encoded.used
         return self._state
 
+    def _bookkeeping(self):
+        return (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len)
+
     def _sync_sizes(self):
-        """Learn from the device how many payload bytes the encodes queued so far have produced (waits for them);
-        raises if one of them failed."""
+        """Learn from the device how many payload bytes the encodes queued so far have produced (waits for them).  If
+        one of them failed, every store queued since the last one known to be good is taken back (their tokens return
+        to the front of the tail) and the error is raised."""
         if self._enc_pending == 0:
             return
-        self._enc_pending = 0
-        _, max_tile, max_stream, _ = kvcomp_cuda.encode_result(self._state[:8], self._encoded.data.numel())
-        self._encoded.used = int(self._state[8].item())
+        self.waits += 1
+        try:
+            _, max_tile, max_stream, _ = kvcomp_cuda.encode_result(self._state[:8], self._encoded.data.numel())
+        except KvcompError:
+            self._roll_back()
+            raise
+        self._probe = None
+        self._accept(len(self._unverified), int(self._state[8].item()), max_tile, max_stream)
+
+    def _accept(self, n_stores: int, used: int, max_tile: int, max_stream: int):
+        """The first n_stores queued stores are done and good; `used` payload bytes lie in _encoded behind them."""
+        done, self._unverified = self._unverified[:n_stores], self._unverified[n_stores:]
+        self._encoded.used = used
+        self._enc_pending = sum(u[3] for u in self._unverified)
         self.max_tile_bytes = max(self.max_tile_bytes, max_tile)
         self.max_stream_bytes = max(self.max_stream_bytes, max_stream)
+        if done:
+            self._verified = done[-1][2] + (used,)
+        if self._trim_after_sync and not self._unverified:
+            self._trim_after_sync = False
+            self._encoded.trim()                               # a byte per symbol was reserved; the stream is a fraction of it
+
+    def _roll_back(self):
+        """Back to the last store that is known to be good: the stores queued since then are dropped from the
+        bookkeeping, the device's words say so too, and the tokens of those stores return to the front of the tail
+        (rows that were not kept -- stores recorded into a graph -- are lost and leave ctx_len)."""
+        if self._verified is None:
+            return
+        (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len,
+         self._encoded.used) = self._verified
+        st = self._state
+        st[1:5] = 0                                            # no error; the size hints start again from the host's
+        st[4] = self._block_infos.used // 8
+        st[8] = self._encoded.used
+        self._enc_pending = 0
+        rows = [u[1] for u in self._unverified if u[1] is not None]
+        self.ctx_len -= sum(u[0] for u in self._unverified if u[4])
+        if rows:
+            if self._tail_len:
+                rows.append(self._tail[:self._tail_len])
+            self._tail = torch.cat(rows, dim=0)
+            self._tail_len = self._tail.shape[0]
+        self._unverified = []
+        self._probe = None
+
+    def _issue_probe(self):
+        """Ask for a copy of the device words without waiting for it (nothing is asked for while the stream is being
+        recorded into a graph, or while an earlier copy is on its way)."""
+        if self._probe is not None or not self._unverified or torch.cuda.is_current_stream_capturing():
+            return
+        if self._host_words is None:
+            self._host_words = torch.empty(16, dtype=torch.int32, pin_memory=True)
+        self._host_words.copy_(self._state, non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        self._probe = (ev, len(self._unverified))
+
+    def poll_stores(self):
+        """Look, without waiting, at what the stores queued by async_store have left: sizes and size hints are brought
+        up to date, and a store that failed on the device is reported here (KvcompError) with the context rolled back to
+        the last good store.  Called by store() and by the attention operator; cheap when nothing is outstanding."""
+        p = self._probe
+        if p is None or not p[0].query():
+            return
+        w = self._host_words
+        if int(w[1]) != 0:
+            self._sync_sizes()                                 # takes the stores back and raises, with the library's message
+            return
+        self._probe = None
+        self._accept(p[1], int(w[8]), int(w[2]), int(w[3]))
+        self._issue_probe()
 
     def encoded_nosync(self):
         """(payload buffer, upper bound of the bytes in use) without waiting for queued encodes: for callers that
@@ -306,6 +387,8 @@ class KVCompCtx:
         if self.device is None:
             self.device = cache.device
         assert self.device == cache.device, "device mismatch"
+        if self._probe is not None:
+            self.poll_stores()
         # cut_tensor_ctx_len_0 (utils/compute.py:59-72): the leading whole blocks of (tail + new tokens) that leave the
         # recent window are compressed, the rest is the new tail.  The blocks are taken from where they lie (the tail,
         # the incoming tensor, or -- when they span both -- a copy of just those tokens), so a long prompt never passes
@@ -342,8 +425,19 @@ class KVCompCtx:
         mask = dims_to_mask(self.quant_dims)
         if (not want_symbols and KVCompCtx.fused_store and self.async_store and self.encode_codebook is not None
                 and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
-            self._encode_direct(to_compress.shape[0], cache=to_compress, mask=mask, tables=self.encode_codebook,
-                                table_bytes=self.encode_codebook.numel())
+            T = to_compress.shape[0]
+            capturing = torch.cuda.is_current_stream_capturing()
+            large = T > self.ASYNC_KEEP_BLOCKS * self.block_size
+            # the rows of a small store are kept until the store is seen to have succeeded (a copy: the caller's tensor
+            # and the tail are both overwritten soon); a large one is waited for here, with its rows still in place
+            keep = None if (large or capturing) else to_compress.clone()
+            self._encode_direct(T, cache=to_compress, mask=mask, tables=self.encode_codebook,
+                                table_bytes=self.encode_codebook.numel(), keep=keep, lost_if_dropped=capturing)
+            if large and not capturing:
+                self._trim_after_sync = True
+                self._sync_sizes()
+            else:
+                self._issue_probe()
             return None
         if (not want_symbols and KVCompCtx.fused_store and self.encode_codebook is not None
                 and kvcomp_cuda.store_fused_supported(self.is_k, mask, self.batch_size, self.head_num, self.head_dim)):
@@ -384,12 +478,16 @@ class KVCompCtx:
     device_codebook = True
     # With a codebook in place, store(want_symbols=False) queues the fused quantize + encode and returns without
     # waiting for it: sizes and errors are learnt the next time something asks for them (encoded_data, get_cr, ...),
-    # and a store that fails on the device is only reported then -- with its metadata already appended.  The caches
-    # that models use switch it on, together with codebook_smoothing, which rules out symbols without a code.
+    # and a store that fails on the device is reported by the next store() or attention call that finds its outcome
+    # (poll_stores: no wait), or by whatever waits for sizes: the context is then rolled back to the last good store,
+    # with the failed stores' tokens back in the tail.  The caches that models use switch it on, together with
+    # codebook_smoothing, which rules out symbols without a code.
     async_store = False
+    # stores of up to this many blocks are queued without a wait; longer ones (a second chunk of a prompt) are waited for
+    ASYNC_KEEP_BLOCKS = 8
 
     def _encode_direct(self, T: int, *, tables, table_bytes, symbols=None, cache=None, mask=0, meta=None,
-                       min_ints=None, quant_scale=None):
+                       min_ints=None, quant_scale=None, keep=None, lost_if_dropped=False):
         """Queue one encode whose outputs go straight to their final places in this context's buffers; nothing waits.
         Quantizes `cache` on the fly (fused store) or takes `symbols` with their min_ints / quant_scale."""
         nb = T // self.block_size
@@ -397,6 +495,9 @@ class KVCompCtx:
         sizes = kvcomp_cuda.buffer_sizes(T, B * H * D, self.is_k, H, D)
         gshape = mask_keepdim_shape((nb, self.block_size, B, H, D), dims_to_mask(self.quant_dims))
         state = self._device_state()
+        if not self._unverified:
+            self._sync_sizes()                                 # (a no-op unless sizes are outstanding for another reason)
+            self._verified = self._bookkeeping() + (self._encoded.used,)
         bi = self._block_infos.reserve(sizes[0], (), torch.uint8, self.device)
         ti = self._thread_infos.reserve(sizes[1], (), torch.uint8, self.device)
         mn = self._min_ints.reserve(nb, gshape[1:], torch.int8, self.device)
@@ -419,6 +520,7 @@ class KVCompCtx:
         self._scales.used += nb
         self._enc_pending += worst
         self.compressed_ctx_len += T
+        self._unverified.append((T, keep, self._bookkeeping(), worst, lost_if_dropped))
 
     def _first_chunk_on_device(self, quant_ints, min_ints, quant_scale):
         """Codebook of the first stored chunk (kvcomp_encode.py:99-103) and its encode, queued back to back on the
@@ -428,23 +530,19 @@ class KVCompCtx:
         if self.codebook_smoothing:
             counts[0, :self._smoothed_symbols()] += 1
         T = quant_ints.shape[0] * quant_ints.shape[1]
-        before = (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len)
         for fmt in (kvcomp_cuda.TREE_I8, kvcomp_cuda.TREE_I16):
             enc, trees, meta = kvcomp_cuda.build_codebook_device(counts, fmt)
             self._encode_direct(T, tables=enc, table_bytes=enc.shape[1], symbols=quant_ints, meta=meta, min_ints=min_ints,
                                 quant_scale=quant_scale)
+            self._trim_after_sync = True                       # a byte per symbol was reserved
             try:
-                self._sync_sizes()
+                self._sync_sizes()                             # (a failure leaves the context as it was before the encode)
                 break
-            except Exception:
-                (self._block_infos.used, self._thread_infos.used, self._min_ints.used, self._scales.used, self.compressed_ctx_len) = before
-                self._state[1] = 0                             # the error has been reported; the context is as it was
-                self._enc_pending = 0
+            except KvcompError:
                 # status 4: the code does not fit the int8 tree (kvc_build_codebook_device) -- once more with the wide one
                 if fmt == kvcomp_cuda.TREE_I8 and int(meta[0, 3]) == 4:
                     continue
                 raise
-        self._encoded.trim()                                   # a byte per symbol was reserved; the stream is a fraction of it
         shift, enc_bytes, dec_bytes, status = (int(v) for v in meta[0].cpu())
         assert status == 0 and shift == 0, "shift must be 0"
         self._set_codebook(enc[0, :enc_bytes].cpu(), trees[0, :dec_bytes].cpu(), tree_format=fmt)

@@ -164,9 +164,9 @@ def test_store_without_waiting_gives_the_same_stream(k_mode):
     B, H, D = 2, 2, 128
     (k_sync, k_async), (v_sync, v_async) = _pair_of_contexts(300, 400, B, H, D, k_mode)
     q = S.synth_q(B, 2 * H, D).to(DEV)
-    assert k_async._enc_pending > 0 and v_async._enc_pending > 0           # nobody has asked for a size yet
+    assert k_async.waits == 1 and v_async.waits == 1                       # the first chunk's codebook; no store since has waited
     out_async = CompressedAttention(k_async, v_async).attend(q)            # an address and a bound are enough
-    assert k_async._enc_pending > 0
+    assert k_async.waits == 1 and v_async.waits == 1
     out_sync = CompressedAttention(k_sync, v_sync).attend(q)
     assert torch.equal(out_async, out_sync)
     for a, b in ((k_sync, k_async), (v_sync, v_async)):
@@ -212,6 +212,8 @@ def test_append_and_attend_can_be_captured_in_a_graph():
     out = torch.empty(B, Hq, D, dtype=torch.float32, device=DEV)
     att.attend(q, out=out)                                   # decode tables and workspace exist before the capture
     # one eager step makes every buffer as large as the step needs; then the host's view is put back
+    for c in (kc, vc):
+        c._sync_sizes()                                       # nothing outstanding: the host's view is exact
     saved = [(c._device_state().clone(), c._encoded.used, c._block_infos.used, c._thread_infos.used, c._min_ints.used,
               c._scales.used, c.compressed_ctx_len, c.ctx_len, c._tail_len, c._enc_pending) for c in (kc, vc)]
     kc.store(k[T0:], want_symbols=False)
@@ -224,6 +226,7 @@ def test_append_and_attend_can_be_captured_in_a_graph():
             c._state.copy_(sv[0])
             (c._encoded.used, c._block_infos.used, c._thread_infos.used, c._min_ints.used, c._scales.used,
              c.compressed_ctx_len, c.ctx_len, c._tail_len, c._enc_pending) = sv[1:]
+            c._unverified, c._probe = [], None
 
     def step():
         rewind()
@@ -342,3 +345,97 @@ def test_one_pass_runs_of_two_over_odd_tile_counts(is_k, T, B, H, D, from_symbol
     second = got_bi[bi.size:2 * bi.size].view(np.uint32).reshape(-1, 2)
     first = bi.view(np.uint32).reshape(-1, 2)
     assert np.array_equal(second[:, 0], first[:, 0] + pay.size) and np.array_equal(second[:, 1], first[:, 1])
+
+
+def test_a_queued_store_that_fails_is_reported_without_a_wait_and_taken_back():
+    """async_store with codebook smoothing off: a block that needs a symbol the first chunk's codebook has no code for
+    fails on the device, after store() has returned.  The next store() or attention call that finds the outcome (no
+    wait) raises, and the context is then what it was after the last good store: bookkeeping, device words and
+    payload position rolled back, the failed block's tokens back in front of the tail, nothing lost."""
+    from kvcomp_amd._lib import KvcompError
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="BlockQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    B, H, D = 1, 2, 128
+    flat = torch.zeros(256, B, H, D, dtype=torch.float16, device=DEV)
+    flat[::2] = 1.0                                               # two symbols only: 0 and 10
+    wide = S.synth_k(64, B, H, D).to(DEV)                         # needs the symbols in between
+    ctx = KVCompCtx(True, B, H, D, 0.1)
+    ctx.async_store = True
+    ctx.store(flat, want_symbols=False)                           # first chunk: codebook of two symbols
+    ctx.store(flat[:64], want_symbols=False)                      # a good block, queued
+    torch.cuda.synchronize()
+    ctx.poll_stores()                                             # its outcome has arrived: known to be good, no wait
+    assert ctx.waits == 1 and not ctx._unverified and ctx.compressed_ctx_len == 320
+    good = (ctx.compressed_ctx_len, ctx.block_infos.numel(), ctx.thread_infos.numel(), ctx.quant_scales.numel(),
+            ctx.encoded_data.numel(), ctx.max_tile_bytes)
+    payload = ctx.encoded_data.clone()
+    ctx.store(wide, want_symbols=False)                           # fails on the device; store() cannot know yet
+    assert ctx.compressed_ctx_len == 384
+    one = torch.full((1, B, H, D), 0.5, dtype=torch.float16, device=DEV)
+    taken = 0
+    with pytest.raises(KvcompError, match="no code"):
+        for _ in range(3):                                        # the outcome arrives some microseconds later
+            ctx.store(one, want_symbols=False)                    # finds it, if it is there, before it does anything else
+            taken += 1
+            torch.cuda.synchronize()
+    assert taken <= 1 and ctx.waits == 2                          # (the one wait that fetched the library's message)
+    assert good == (ctx.compressed_ctx_len, ctx.block_infos.numel(), ctx.thread_infos.numel(), ctx.quant_scales.numel(),
+                    ctx.encoded_data.numel(), ctx.max_tile_bytes)
+    assert torch.equal(ctx.encoded_data, payload)
+    assert ctx.ctx_len == 384 + taken and ctx.buffer.shape[0] == 64 + taken      # the store that raised took nothing in
+    assert torch.equal(ctx.buffer[:64], wide) and torch.equal(ctx.buffer[64:], one[:taken])
+    assert ctx._state[:5].tolist() == [ctx._state[0].item(), 0, 0, 0, ctx.block_infos.numel() // 8] and int(ctx._state[8]) == payload.numel()
+    full, _ = ctx.get()
+    assert torch.equal(full[:320], torch.cat([flat, flat[:64]])) and torch.equal(full[320:], ctx.buffer)
+    # the block that cannot be encoded is still in the tail, so the next store that reaches a block boundary fails the same way
+    with pytest.raises(KvcompError, match="no code"):
+        for _ in range(200):
+            ctx.store(one, want_symbols=False)
+            torch.cuda.synchronize()
+    assert ctx.compressed_ctx_len == 320 and torch.equal(ctx.encoded_data, payload)
+
+
+def test_a_second_prompt_chunk_leaves_no_worst_case_reservation_behind():
+    """A long store into a context that has its codebook reserves a byte per symbol for the payload; the reservation
+    is given back once the sizes are known, so the context holds little more than its stream."""
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    T, B, H, D = 4096, 2, 4, 128
+    for is_k in (True, False):
+        x = (S.synth_k if is_k else S.synth_v)(2 * T, B, H, D).to(DEV)
+        ctx = KVCompCtx(is_k, B, H, D, 0.1 if is_k else 0.2)
+        ctx.codebook_smoothing = True
+        ctx.async_store = True
+        ctx.store(x[:T], want_symbols=False)
+        ctx.store(x[T:], want_symbols=False)                      # waited for: longer than ASYNC_KEEP_BLOCKS blocks
+        assert ctx.compressed_ctx_len >= 2 * T - 128 and not ctx._unverified
+        tail_bytes = ctx._tail.numel() * 2
+        assert ctx.held_bytes() - tail_bytes <= 1.5 * ctx.compressed_bytes(), (ctx.held_bytes(), ctx.compressed_bytes())
+        twin = KVCompCtx(is_k, B, H, D, 0.1 if is_k else 0.2)
+        twin.codebook_smoothing = True
+        twin.store(x[:T], want_symbols=False)
+        twin.store(x[T:], want_symbols=False)
+        assert torch.equal(ctx.encoded_data, twin.encoded_data) and torch.equal(ctx.block_infos, twin.block_infos)
+
+
+def test_size_hints_follow_queued_stores_without_a_wait():
+    """The largest tile and the longest stream (which size the fused decoders' LDS areas) are brought up to date from
+    the copies of the device words that arrive behind queued stores: no wait, and no stale hints over a long decode."""
+    from kvcomp_amd.ctx import KVCompCtx
+    _config(k_mode="ChannelQuant", v_mode="TokenQuant", k_recent=64, v_recent=128)
+    B, H, D = 2, 2, 128
+    quiet = (S.synth_k(256, B, H, D) * 0.0 + S.synth_k(256, B, H, D, 5).sign()).to(torch.float16).to(DEV)   # two levels per channel
+    busy = S.synth_k(256, B, H, D, 6).to(DEV)
+    a, b = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(True, B, H, D, 0.1)
+    for c in (a, b):
+        c.codebook_smoothing = True
+    a.async_store = True
+    for c in (a, b):
+        c.store(quiet, want_symbols=False)                        # small tiles first
+        for i in range(256):
+            c.store(busy[i:i + 1], want_symbols=False)            # larger ones later
+    torch.cuda.synchronize()
+    a.poll_stores()
+    assert a.waits == 1
+    assert (a.max_tile_bytes, a.max_stream_bytes) == (b.max_tile_bytes, b.max_stream_bytes)
+    assert a.max_tile_bytes > 0 and a._enc_pending == 0
