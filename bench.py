@@ -219,6 +219,27 @@ def measured_traffic(workload, kernel):
     return t.get("bytes_per_launch", {}).get(workload, {}).get(kernel)
 
 
+def check_layer_attention(attn, q, tokens):
+    """One layer's decode attention against fp32 attention over the dequantized cache (compressed part + fp16 tail, as
+    KVCompCtx.get() returns it), a batch entry at a time; returns the largest error relative to max|reference| and
+    raises beyond the 1e-3 this path is held to."""
+    import torch
+    kctx, vctx = attn.k, attn.v
+    out = attn.attend(q)
+    kd, vd = kctx.get()[0], vctx.get()[0]
+    assert kd.shape[0] == vd.shape[0] == tokens
+    B, Hq, D = q.shape
+    rep = Hq // kctx.head_num
+    worst = 0.0
+    for b in range(B):
+        kb, vb = kd[:, b].float().repeat_interleave(rep, dim=1), vd[:, b].float().repeat_interleave(rep, dim=1)
+        s = torch.einsum("thd,hd->ht", kb, q[b].float()) / D ** 0.5
+        ref = torch.einsum("ht,thd->hd", torch.softmax(s, dim=-1), vb)
+        worst = max(worst, float((out[b] - ref).abs().max() / ref.abs().max()))
+    assert worst <= 1e-3, "decode attention differs from fp32 attention over the dequantized cache by %.2e" % worst
+    return worst
+
+
 def run_decode_loop(args, emit=True):
     """cfg4 without the model around it: every layer of a Llama-2-7B-shaped stack keeps a compressed K and V cache;
     a step appends one new token per sequence to every layer (compressing the 64- / 128-token blocks that leave
@@ -269,6 +290,9 @@ def run_decode_loop(args, emit=True):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     assert torch.isfinite(out).all()
+    # after the timed steps: two layers' operators against fp32 attention over what their caches hold now
+    check_err = max(check_layer_attention(layers[l][2], q[l], layers[l][0].ctx_len) for l in (0, L - 1))
+    log("[bench] cfg4 cache loop checked against fp32 attention over the dequantized cache (layers 0 and %d): max error %.1e" % (L - 1, check_err))
     comp = sum(k.compressed_bytes() + v.compressed_bytes() for k, v, _ in layers)
     tails = sum((k.buffer.numel() + v.buffer.numel()) * 2 for k, v, _ in layers)
     tokens = layers[0][0].ctx_len
@@ -282,7 +306,7 @@ def run_decode_loop(args, emit=True):
                    "cache_bytes": {"compressed": comp, "fp16_tails": tails, "fp16_equivalent": raw},
                    "compression_ratio_whole_cache": round(raw / (comp + tails), 3),
                    "compression_ratio_compressed_part": {"k": round(layers[0][0].get_cr(), 3), "v": round(layers[0][1].get_cr(), 3)},
-                   "prefill_compress_s": round(t_prefill, 3),
+                   "prefill_compress_s": round(t_prefill, 3), "check_max_error": check_err,
                    "not_run": "projections, MLP, norms, sampling (outside this path)"},
         "roofline": None, "cpu_baseline": None,
     }
@@ -383,7 +407,8 @@ def other_configs(args):
     loop = run_decode_loop(types.SimpleNamespace(steps=20, warmup=5, sync_store=False), emit=False)
     res["cfg4_cache_loop"] = {"workload": loop["config"]["workload"], "ms_per_step": loop["ms_per_step"], "tokens_per_s": loop["value"],
                               "steps": loop["steps"], "compression_ratio_whole_cache": loop["config"]["compression_ratio_whole_cache"],
-                              "prefill_compress_s": loop["config"]["prefill_compress_s"], "not_run": loop["config"]["not_run"]}
+                              "prefill_compress_s": loop["config"]["prefill_compress_s"], "check_max_error": loop["config"]["check_max_error"],
+                              "not_run": loop["config"]["not_run"]}
     log("[bench] cfg4 cache loop: %.2f ms per step, %.0f tokens/s" % (loop["ms_per_step"], loop["value"]))
     # cfg4 with the model around the cache (random weights), and the same model on transformers' dense fp16 cache
     try:
@@ -397,7 +422,7 @@ def other_configs(args):
         model[key] = {"tokens_per_s": r["value"], "ms_per_step": r["ms_per_step"], "steps": r["steps"],
                       "prefill_s": r["config"]["prefill_s"], "cache_bytes_held": r["config"]["cache_bytes_held"],
                       "compression_ratio_whole_cache": r["config"]["compression_ratio_whole_cache"],
-                      "attention": r["config"]["attention"]}
+                      "check_max_error": r["config"]["check_max_error"], "attention": r["config"]["attention"]}
         log("[bench] cfg4 model, %s: %.2f ms per step, %.0f tokens/s" % (key.replace("_", " "), r["ms_per_step"], r["value"]))
     model["workload"] = "Llama-2-7B architecture (stock transformers code, random fp16 weights), 32 layers, batch 8, 4096-token random prompt, 64 greedy tokens"
     res["cfg4_model"] = model
@@ -456,6 +481,16 @@ def run_model_decode(args, emit=True):
             nxt = model(nxt, past_key_values=cache, use_cache=True).logits[:, -1].argmax(-1, keepdim=True)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
+    check_err = None
+    if not args.dense_cache:
+        # the first and the last layer's streams as generation left them: the operator the model attended with against
+        # fp32 attention over the dequantized cache, with a fresh random query
+        from kvcomp_amd.attention import CompressedAttention
+        gq = torch.Generator().manual_seed(1236)
+        qs = torch.randn(B, H, D, generator=gq, dtype=torch.float32).to(torch.float16).to(dev)
+        check_err = max(check_layer_attention(CompressedAttention(cache.layers[l].k_ctx, cache.layers[l].v_ctx), qs,
+                                              cache.get_seq_length()) for l in (0, L - 1))
+        log("[bench] cfg4 model: layers 0 and %d checked against fp32 attention over the dequantized cache: max error %.1e" % (L - 1, check_err))
     result = {
         "metric": "decode tokens/s, Llama-2-7B architecture (random weights) with a compressed KV cache in every layer",
         "value": round(B * args.new_tokens / dt, 2), "unit": "tokens/s", "n_gpus": 1, "steps": args.new_tokens,
@@ -467,7 +502,7 @@ def run_model_decode(args, emit=True):
                    "compression_ratio_whole_cache": None if args.dense_cache else round(cache.compression_ratio(), 3),
                    "cache_bytes_held": (2 * 2 * L * cache.get_seq_length() * B * H * D if args.dense_cache
                                         else cache.compressed_bytes()),
-                   "prefill_s": round(t_prefill, 3),
+                   "prefill_s": round(t_prefill, 3), "check_max_error": check_err,
                    "attention": ("transformers DynamicCache (dense fp16) and stock SDPA: the comparison run" if args.dense_cache else
                                  "single-token steps: kvc_attention_decode on the compressed streams; prompt: stock SDPA")},
         "roofline": None, "cpu_baseline": None,

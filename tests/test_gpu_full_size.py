@@ -113,3 +113,63 @@ def test_full_size_round_trip_and_attention(name):
     assert float((out_rf.double() - ref_fp16).abs().max()) <= 1e-3 * scale
     # ... element by element too: within 1e-3 of the value, or of the output's typical size for the smallest ones
     assert torch.allclose(out_r.double(), ref_fp16, rtol=1e-3, atol=1e-3 * float(ref_fp16.pow(2).mean().sqrt()))
+
+
+def test_cfg4_layer_at_its_own_shape_through_the_append_loop():
+    """One layer of the full-decode configuration at its own shape: batch 8, 32 heads x 128, a 4096-token prompt and
+    130 appended tokens through KVCompCtx as the model-facing caches set it up (stores queued without a wait, codebook
+    smoothing), K recompressing every 64 and V every 128 tokens.  After tokens 1, 64, 65, 128, 129 and 130 the
+    attention operator (compressed part + fp16 tails) must match float64 attention over get() within 1e-3, and the
+    queued stores must have produced the stream of a context that waits for every store.  Reference contract:
+    models/cache/kvcomp_encode.py:345-360 (update), models/llama.py:279-304 (attention over what update returns)."""
+    from kvcomp_amd.attention import CompressedAttention
+    from kvcomp_amd.compute import QuantMode
+    from kvcomp_amd.ctx import KVCompCacheConfig, KVCompCacheConfigStatic, KVCompCtx
+    B, H, D, T, NEW = 8, 32, 128, 4096, 130
+    KVCompCacheConfigStatic.config = KVCompCacheConfig("cfg4", QuantMode.ChannelQuant, QuantMode.TokenQuant, 64, 128, 64, 128, 0.1, 0.2)
+    import bench
+    cfg = dict(B=B, H=H, Hq=H, D=D, T=T + 192, eb_k=0.1, eb_v=0.2, dist="gauss")
+    k, v = bench.make_kv(cfg, torch.device(DEV))
+    g = torch.Generator(device=DEV).manual_seed(1236)
+    ctxs = {}
+    for name, asynchronous in (("queued", True), ("waiting", False)):
+        kc, vc = KVCompCtx(True, B, H, D, 0.1), KVCompCtx(False, B, H, D, 0.2)
+        for c in (kc, vc):
+            c.codebook_smoothing = True
+            c.async_store = asynchronous
+        kc.store(k[:T], want_symbols=False)
+        vc.store(v[:T], want_symbols=False)
+        ctxs[name] = (kc, vc)
+    kc, vc = ctxs["queued"]
+    attn = CompressedAttention(kc, vc)
+
+    def check(step):
+        q = torch.randn(B, H, D, generator=g, device=DEV, dtype=torch.float32).to(torch.float16)
+        out = attn.attend(q)
+        kd, vd = kc.get()[0], vc.get()[0]                               # [T, B, H, D] fp16: compressed part + tail
+        assert kd.shape[0] == vd.shape[0] == T + step
+        worst = 0.0
+        for b in range(B):                                              # a batch entry at a time keeps float64 small
+            s = torch.einsum("thd,hd->ht", kd[:, b].double(), q[b].double()) / math.sqrt(D)
+            ref = torch.einsum("ht,thd->hd", torch.softmax(s, dim=-1), vd[:, b].double())
+            scale = float(ref.abs().max())
+            worst = max(worst, float((out[b].double() - ref).abs().max()) / scale)
+            assert torch.allclose(out[b].double(), ref, rtol=1e-3, atol=1e-3 * float(ref.pow(2).mean().sqrt()))
+        assert worst <= 1e-3, (step, worst)
+        return worst
+
+    check(0)
+    seen = set()
+    for i in range(NEW):
+        for name in ("queued", "waiting"):
+            ctxs[name][0].store(k[T + i:T + i + 1], want_symbols=False)
+            ctxs[name][1].store(v[T + i:T + i + 1], want_symbols=False)
+        if i + 1 in (1, 64, 65, 128, 129, 130):
+            check(i + 1)
+            seen.add((kc.compressed_ctx_len, vc.compressed_ctx_len))
+    assert len(seen) >= 3                                               # the checks saw K and V recompress
+    assert kc.waits == 1 and vc.waits == 1                              # nothing since the prompt's codebook has waited
+    for a, b in zip(ctxs["queued"], ctxs["waiting"]):
+        assert a.compressed_ctx_len == b.compressed_ctx_len > T - 128 and a.ctx_len == b.ctx_len == T + NEW
+        for name in ("encoded_data", "block_infos", "thread_infos", "quant_min_ints", "quant_scales", "buffer"):
+            assert torch.equal(getattr(a, name), getattr(b, name)), name
