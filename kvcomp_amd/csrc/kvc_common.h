@@ -58,7 +58,7 @@ constexpr int KVC_TREE_MAX_NODES = 512;                   // 2 * 256 symbols - 2
 // ---------------------------------------------------------------------------------------------------
 int kvc_fail(int code, const char *fmt, ...);
 // Tuning knobs settable through kvc_set_option (or, before first use, KVCOMP_<NAME> in the environment).
-enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_DECODE_PIPELINED = 5, KVC_OPT_FUSED_ROUNDED = 6, KVC_OPT_ATTENTION_TAIL_IN_MERGE = 7, KVC_OPT_FUSED_MFMA = 8, KVC_OPT_FUSED_BUILTIN_DPP = 9, KVC_OPT_FUSED_SCHEDULE = 10, KVC_OPT_ENCODE_ONE_PASS = 11, KVC_OPT_FUSED_HALF_TABLE = 12, KVC_OPT_ENCODE_LOOKBACK_POLLS = 13, KVC_OPT_COUNT };
+enum KvcOption { KVC_OPT_FUSED_ROWS = 0, KVC_OPT_FUSED_TILES_PER_WAVE = 1, KVC_OPT_FUSED_PAIR_BITS = 2, KVC_OPT_FUSED_DOUBLE_WINDOW = 3, KVC_OPT_FUSED_SKEW = 4, KVC_OPT_DECODE_PIPELINED = 5, KVC_OPT_FUSED_ROUNDED = 6, KVC_OPT_ATTENTION_TAIL_IN_MERGE = 7, KVC_OPT_FUSED_MFMA = 8, KVC_OPT_FUSED_BUILTIN_DPP = 9, KVC_OPT_FUSED_SCHEDULE = 10, KVC_OPT_ENCODE_ONE_PASS = 11, KVC_OPT_FUSED_HALF_TABLE = 12, KVC_OPT_ENCODE_LOOKBACK_POLLS = 13, KVC_OPT_FUSED_SCHEDULE_V = 14, KVC_OPT_FUSED_TILES_PER_WAVE_V = 15, KVC_OPT_COUNT };
 int kvc_option(KvcOption which);
 int kvc_check_hip(hipError_t e, const char *what);
 // A slot of the per-device scratch ring (each slot holds KVC_WS_SLOT_BYTES); used for the LUT that the

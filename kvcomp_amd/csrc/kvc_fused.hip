@@ -910,14 +910,20 @@ static size_t kvc_plan_lds(KvcFusedArgs &a, int slots, int rep, int64_t encoded_
 // Consecutive tiles of a row that one wave works through (fetching one ahead): as many as still leave
 // every SIMD of the chip several waves.
 constexpr int KVC_DEFAULT_SCHEDULE = 47020;      // runs of 4 for 70 % of the tiles, of 2 for 20 %, single tiles last
+constexpr int KVC_DEFAULT_SCHEDULE_UNIT3 = 67020; // runs of 6 (two head pairs of head_dim 96), then of 3, single tiles last
 
-static int kvc_plan_tiles_per_wave(int64_t tiles)
+// `unit`: V tiles (matrix-core kernels, rounded arithmetic) after which the heads repeat -- the tiles of one head, or of
+// a pair of heads where head_dim is no multiple of 64 (three tiles over two heads of 96 channels): a wave that takes
+// whole units builds every head's operand tables once.  0: nothing to share (K tiles; the other kernels).
+static int kvc_plan_tiles_per_wave(int64_t tiles, int unit = 0)
 {
-    const int forced = kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE);
+    const int forced_v = unit ? kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE_V) : -1;
+    const int forced = forced_v > 0 ? forced_v : kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE);
     if (forced > 0) return forced > 64 ? 64 : forced;
     // measured on MI355X: two is best once there are enough tiles (the fetch of the second overlaps the
     // decode of the first; 49 152 tiles: 3 % faster than one); at 16 384 tiles one is 3 % faster, and longer runs
     // only leave fewer workgroups to balance over the chip (8 per wave: 15 % slower)
+    if (unit > 1 && unit <= 4 && forced_v < 0 && tiles >= 8192) return unit;
     return tiles >= 32768 ? 2 : 1;
 }
 
@@ -925,14 +931,16 @@ static int kvc_plan_tiles_per_wave(int64_t tiles)
 // first, so that most tiles share a wave's set-up and their fetches overlap the previous tile's decode, shorter ones
 // after, single tiles last, so that the last workgroups to start are short.  Returns the number of workgroups, 0 for
 // the plain 2-D grid.
-static unsigned kvc_plan_schedule(KvcFusedArgs &a, int64_t tiles)
+static unsigned kvc_plan_schedule(KvcFusedArgs &a, int64_t tiles, int unit = 0)
 {
     a.sched_nseg = 0;
     int want = kvc_option(KVC_OPT_FUSED_SCHEDULE);
+    if (unit && kvc_option(KVC_OPT_FUSED_SCHEDULE_V) >= 0) want = kvc_option(KVC_OPT_FUSED_SCHEDULE_V);
     if (want == 0 || a.s.rows_per_codebook != 0 || tiles > (int64_t)1 << 30) return 0;
     if (want < 0) {
         if (tiles < 32768) return 0;      // few tiles: one or two per wave in the plain grid
-        want = KVC_DEFAULT_SCHEDULE;
+        // runs that are whole units (and, halved and quartered, stay whole units or single tiles)
+        want = unit == 3 ? KVC_DEFAULT_SCHEDULE_UNIT3 : KVC_DEFAULT_SCHEDULE;
     }
     const int run0 = want / 10000, pct0 = (want / 100) % 100, pct1 = want % 100;
     if (run0 < 1 || run0 > 64 || pct0 + pct1 > 100) return 0;
@@ -1041,7 +1049,14 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
                             : kvc_plan_lds(a, slots, rounded ? (int)rep + 1 : (int)rep, encoded_bytes, rows * a.s.cols,
                                            max_tile_bytes, max_stream_bytes, max_code_bits, 0, !rounded);
     a.rounded = rounded;
-    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols);
+    // V tiles after which the heads repeat (the kernels that keep a head's operand tables from tile to tile)
+    int unit = 0;
+    if (!is_k && mfma && rounded) {
+        int64_t l = head_dim;
+        while (l % KVC_WAVE != 0) l += head_dim;               // least common multiple of head_dim and 64
+        unit = (int)(l / KVC_WAVE);
+    }
+    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols, unit);
     KvcTimer timer(elapsed_ms, stream);
     if (!d_luts) {
         if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
@@ -1049,7 +1064,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
     dim3 grid = kvc_grid(a.s, rows);
     a.sched_nseg = 0;
     if (mfma) {
-        if (const unsigned wgs = kvc_plan_schedule(a, rows * a.s.cols)) grid = dim3(wgs, 1);
+        if (const unsigned wgs = kvc_plan_schedule(a, rows * a.s.cols, unit)) grid = dim3(wgs, 1);
     }
     static const bool trace_plan = getenv("KVCOMP_TRACE_PLAN") != nullptr;
     if (trace_plan && a.sched_nseg)

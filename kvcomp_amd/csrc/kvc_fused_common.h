@@ -71,7 +71,9 @@ constexpr int kvc_fused_occupancy(int rep, int kind)
 #endif
 constexpr int kvc_fused_mfma_occupancy(int rep, int kind)
 {
-    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : KVC_MFMA_OCC_V1) : kvc_fused_occupancy(rep, kind);
+    // (four query heads, K: the kernel needs 80 registers, which leave six waves; with a bound of five the register
+    // allocator settles on 81 and the sixth wave is lost: 46 -> 49 us at batch 16 x 8 KV heads x 8192 tokens)
+    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : KVC_MFMA_OCC_V1) : (rep == 4 && kind == 0) ? 6 : kvc_fused_occupancy(rep, kind);
 }
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2
@@ -198,12 +200,103 @@ __device__ __forceinline__ T kvc_load_at(const void *uniform_base, uint32_t byte
     return *reinterpret_cast<const T *>(reinterpret_cast<const char *>(uniform_base) + byte_offset);
 }
 
+// Where a tile lies: its row and column in the tile grid and what follows from the column -- the (batch entry, head)
+// it belongs to and, for a V tile, the first of its 64 channels inside that head.  Working these out from the column
+// takes integer divisions, for which the hardware has no scalar instruction (each becomes some fifteen vector
+// instructions, wave-uniform or not); stepping to the next tile of the row-major sequence takes a few scalar additions.
+struct KvcTilePos {
+    int row, col;
+    int b, h;       // K: the tile's (batch entry, kv head); V: those of the tile's first channel
+    int d0;         // V: the first channel's index inside head h (K: 0)
+};
+
+template <bool IS_K>
+__device__ __forceinline__ KvcTilePos kvc_tile_pos(const KvcFusedArgs &a, int row, int col)
+{
+    KvcTilePos p;
+    p.row = row;
+    p.col = col;
+    if (IS_K) {
+        p.b = col / a.kv_heads;
+        p.h = col - p.b * a.kv_heads;
+        p.d0 = 0;
+    } else {
+        const int c0 = col * KVC_WAVE, bh = c0 / a.head_dim;
+        p.d0 = c0 - bh * a.head_dim;
+        p.b = bh / a.kv_heads;
+        p.h = bh - p.b * a.kv_heads;
+    }
+    return p;
+}
+
+template <bool IS_K>
+__device__ __forceinline__ KvcTilePos kvc_tile_after(const KvcFusedArgs &a, KvcTilePos p)
+{
+    p.col++;
+    if (p.col == a.s.cols) {                                // the rows' tiles cover all (batch entry, head) pairs exactly
+        p.col = 0;
+        p.row++;
+        p.b = p.h = p.d0 = 0;
+        return p;
+    }
+    if (IS_K) {
+        p.h++;
+    } else {
+        p.d0 += KVC_WAVE;
+        if (p.d0 < a.head_dim) return p;
+        p.d0 -= a.head_dim;
+        p.h++;
+        while (p.d0 >= a.head_dim) {                        // heads narrower than a tile
+            p.d0 -= a.head_dim;
+            p.h++;
+        }
+    }
+    while (p.h >= a.kv_heads) {
+        p.h -= a.kv_heads;
+        p.b++;
+    }
+    return p;
+}
+
+// (batch entry, head) of a V tile's second head (the one its channels past a head boundary belong to), clamped to the
+// last pair: the tile that ends a row has no second head and must not make one up.
+__device__ __forceinline__ void kvc_second_head(const KvcFusedArgs &a, const KvcTilePos &p, int &b, int &h)
+{
+    b = p.b;
+    h = p.h + 1;
+    if (h == a.kv_heads) {
+        if (b + 1 < a.batch) b++, h = 0;
+        else h = p.h;
+    }
+}
+
 // Issue the global loads of tile (row, col).  bi_off / bi_bn: the tile's block_info words.
-template <int REP, int KIND, int EXPAND = 0>
-__device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
-                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw)
+// Parameters of a V tile's two elements per lane where every token has groups of its own per batch entry (or per batch
+// entry and head): two 2-byte and two 1-byte loads.
+template <class Raw>
+__device__ __forceinline__ void kvc_fetch_separate_params(const KvcFusedArgs &a, int row, int b, int h, int lane, int s, Raw &raw)
+{
+    const int64_t tk0 = (int64_t)row * KVC_V_TOKENS;
+#pragma unroll
+    for (int half = 0; half < 2; half++) {
+        // group of token tk0 + t: (tk0 + t) * batch + b, times kv_heads + h for per-vector groups
+        const int64_t per = a.quant_mask == KVC_MASK_SIM_TOKEN ? a.batch : (int64_t)a.batch * a.kv_heads;
+        const int64_t g0 = a.quant_mask == KVC_MASK_SIM_TOKEN ? tk0 * per + b : tk0 * per + (int64_t)b * a.kv_heads + h;
+        const uint32_t t = 2u * (uint32_t)lane + half;
+        raw.scw[s][half] = kvc_load_at<uint16_t>(a.scale + g0, 2u * t * (uint32_t)per);
+        raw.mnw[s][half] = kvc_load_at<uint8_t>(a.min_i8 + g0, t * (uint32_t)per);
+    }
+}
+
+// `skip_x`: bit s set = the weights of head slot s are not needed (the wave still has that head's operand table).
+// LATE_SECOND: the separate-groups parameters of a tile's second head are left to the caller, who fetches them when the
+// tile is staged (kvc_fetch_separate_params): four registers less to hold through the previous tile's decode loops.
+template <int REP, int KIND, int EXPAND = 0, bool LATE_SECOND = false>
+__device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, const KvcTilePos &pos, uint32_t bi_off, uint32_t bi_bn,
+                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw, int skip_x = 0)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    const int row = pos.row, col = pos.col;
     const int64_t tile = (int64_t)row * a.s.cols + col;                 // wave-uniform, like everything derived from it
     const int D = a.head_dim;
     // sizes are clamped so that corrupt metadata yields wrong symbols, never an out-of-bounds access
@@ -228,7 +321,7 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
     // operands; lanes past the end of a short vector load the last pair (ignored when staged)
     const int mode = kvc_pair_mode<KIND>(a);
     if (KIND == 0) {
-        const int b = col / a.kv_heads, h = col - b * a.kv_heads;
+        const int b = pos.b, h = pos.h;
         const uint32_t e0 = (uint32_t)(2 * lane < D ? 2 * lane : D - 2);
         if (EXPAND != 1) {                                     // symbols out: no quantization parameters
             // per-channel pairs, or one pair per 64-token block (kernels.cu:771-772)
@@ -246,35 +339,29 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
                 raw.x[0][r][0] = kvc_load_at<uint32_t>(a.x + ((int64_t)b * a.q_heads + h * REP + r) * D, 2u * e0);
         }
     } else {
-        const int bh0 = (col * KVC_WAVE) / D;
-        const int bh_max = a.batch * a.kv_heads - 1;
         const int64_t tk0 = (int64_t)row * KVC_V_TOKENS;       // the group's first token; this lane's are tk0 + 2 lane (+ 1)
-        const bool straddles = col * KVC_WAVE - bh0 * D + KVC_WAVE > D;   // wave-uniform
+        const bool straddles = pos.d0 + KVC_WAVE > D;          // wave-uniform
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
             if (s == 1 && !straddles) continue;                // the second head's operands are not needed
-            int bh = bh0 + s;
-            bh = bh < bh_max ? bh : bh_max;                    // slot 1 is unused by a tile that ends the row
-            const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
+            int b = pos.b, h = pos.h;
+            if (s == 1) kvc_second_head(a, pos, b, h);         // (unused by a tile that ends the row)
             if (EXPAND != 1) {
-                if (mode == KVC_PAIR_ADJACENT) {               // one group per token (for this batch entry and head)
-                    raw.scw[s][0] = kvc_load_at<uint32_t>(a.scale + tk0, 4u * (uint32_t)lane);
-                    raw.mnw[s][0] = kvc_load_at<uint16_t>(a.min_i8 + tk0, 2u * (uint32_t)lane);
-                } else {
-#pragma unroll
-                    for (int half = 0; half < 2; half++) {
-                        // group of token tk0 + t: (tk0 + t) * batch + b, times kv_heads + h for per-vector groups
-                        const int64_t per = a.quant_mask == KVC_MASK_SIM_TOKEN ? a.batch : (int64_t)a.batch * a.kv_heads;
-                        const int64_t g0 = a.quant_mask == KVC_MASK_SIM_TOKEN ? tk0 * per + b : tk0 * per + (int64_t)b * a.kv_heads + h;
-                        const uint32_t t = 2u * (uint32_t)lane + half;
-                        raw.scw[s][half] = kvc_load_at<uint16_t>(a.scale + g0, 2u * t * (uint32_t)per);
-                        raw.mnw[s][half] = kvc_load_at<uint8_t>(a.min_i8 + g0, t * (uint32_t)per);
+                if (mode == KVC_PAIR_ADJACENT) {               // one group per token, whatever the batch entry and head:
+                    if (s == 0) {                              // loaded once (also where the first head needs nothing)
+                        raw.scw[0][0] = kvc_load_at<uint32_t>(a.scale + tk0, 4u * (uint32_t)lane);
+                        raw.mnw[0][0] = kvc_load_at<uint16_t>(a.min_i8 + tk0, 2u * (uint32_t)lane);
+                    } else {
+                        raw.scw[s][0] = raw.scw[0][0];
+                        raw.mnw[s][0] = raw.mnw[0][0];
                     }
+                } else if (!((skip_x >> s) & 1) && (s == 0 || !LATE_SECOND)) {
+                    kvc_fetch_separate_params(a, row, b, h, lane, s, raw);
                 }
             }
 #pragma unroll
             for (int r = 0; r < REP; r++) {
-                if (EXPAND != 0) break;
+                if (EXPAND != 0 || ((skip_x >> s) & 1)) break;
                 const int64_t xrow = (int64_t)b * a.q_heads + h * REP + r;
                 if (KvcGeom<KIND>::SOFTMAX) {
                     const uint2 v = kvc_load_at<uint2>(a.scores + xrow * a.scores_stride + tk0, 8u * (uint32_t)lane);
@@ -286,6 +373,14 @@ __device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, i
             }
         }
     }
+}
+
+// The same for callers that know the tile by its row and column only.
+template <int REP, int KIND, int EXPAND = 0>
+__device__ __forceinline__ void kvc_fetch_tile(const KvcFusedArgs &a, int row, int col, uint32_t bi_off, uint32_t bi_bn,
+                                               int lane, KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw)
+{
+    kvc_fetch_tile<REP, KIND, EXPAND>(a, kvc_tile_pos<KIND == 0>(a, row, col), bi_off, bi_bn, lane, raw);
 }
 
 __device__ __forceinline__ float kvc_half_bits_to_float(uint32_t bits16)

@@ -133,23 +133,98 @@ __device__ __forceinline__ void kvc_mfma_min_scale_words(const Raw &raw, int s, 
     }
 }
 
-// Build the operand tables of a fetched tile; returns per query head the constant term sum_i min_i weight_i of this
-// lane's head slot (zero in rounded mode) and the power of two the weights were divided by to stay inside fp16.
+// Which of the wave's operand-table slots serve a tile.  A V tile needs the tables of one head, or of two when its 64
+// channels straddle a head boundary; consecutive tiles of a row share heads (head_dim 128: two tiles per head;
+// head_dim 96: three tiles over two heads), and a head's tables -- the softmax of its 128 scores, the weights split into
+// fp16 parts, the tokens' minima and scales -- are the same for every tile.  So a wave that works through a run of tiles
+// keeps what it has built: KvcTableState says which head each slot holds, kvc_plan_tables which slot a tile's first head
+// uses (the second head's is the other one) and which heads still have to be built.  Rounded mode only (the other
+// arithmetic folds per-tile constants into its tables); K tiles change head, or block of channel parameters, every tile.
+// (Plain integers picked with selects, no arrays: an array indexed by a run-time slot number would live in scratch memory.)
+struct KvcTableState {
+    int head0, head1;         // batch entry * kv_heads + head whose tables lie in slot 0 / 1, -1: none
+    int row;                  // tile row they were built for
+    int lo0, lo1;             // the slot's low-part columns hold something
+    __device__ __forceinline__ int head(int slot) const { return slot ? head1 : head0; }
+    __device__ __forceinline__ int lo(int slot) const { return slot ? lo1 : lo0; }
+    __device__ __forceinline__ void set_head(int slot, int h)
+    {
+        head0 = slot ? head0 : h;
+        head1 = slot ? h : head1;
+    }
+    __device__ __forceinline__ void set_lo(int slot, int v)
+    {
+        lo0 = slot ? lo0 : v;
+        lo1 = slot ? v : lo1;
+    }
+};
+
+struct KvcTablePlan {
+    int slot0;                // table slot of the tile's first head
+    int build;                // bit s set: head s of the tile (0: first, 1: second) has to be built
+    int straddles;
+};
+
+template <int KIND, bool ROUNDED>
+__device__ __forceinline__ KvcTablePlan kvc_plan_tables(const KvcFusedArgs &a, const KvcTilePos &p, KvcTableState &st)
+{
+    constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
+    KvcTablePlan pl;
+    pl.slot0 = 0;
+    pl.straddles = (SLOTS == 2 && p.d0 + KVC_WAVE > a.head_dim) ? 1 : 0;
+    pl.build = pl.straddles ? 3 : 1;
+    if constexpr (KIND != 0 && ROUNDED) {
+        const bool same_row = st.row == p.row;
+        const int hA = p.b * a.kv_heads + p.h;
+        if constexpr (SLOTS == 1) {
+            if (same_row && st.head0 == hA) pl.build = 0;
+            st.head0 = hA;
+        } else {
+            int b2, h2;
+            kvc_second_head(a, p, b2, h2);
+            const int hB = pl.straddles ? b2 * a.kv_heads + h2 : -2;
+            const bool in0 = same_row && st.head0 == hA, in1 = same_row && st.head1 == hA;
+            const bool buildA = !in0 && !in1;
+            // a head that has to be built leaves the second head's tables where they are
+            const int sA = in0 ? 0 : in1 ? 1 : (same_row && st.head0 == hB) ? 1 : 0;
+            const int sB = 1 - sA;
+            const bool buildB = pl.straddles && !(same_row && st.head(sB) == hB);
+            pl.slot0 = sA;
+            pl.build = (buildA ? 1 : 0) | (buildB ? 2 : 0);
+            if (!same_row) st.head0 = st.head1 = -1;
+            st.set_head(sA, hA);
+            if (pl.straddles) st.set_head(sB, hB);
+        }
+        st.row = p.row;
+    }
+    return pl;
+}
+
+// Build those operand tables of a fetched tile that the plan asks for; returns per query head the constant term
+// sum_i min_i weight_i of this lane's head (zero in rounded mode) and the power of two the weights were divided by to
+// stay inside fp16; sel_out: 1 for a lane whose channel lies past the tile's head boundary.
 template <int REP, int KIND, bool ROUNDED>
-__device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int row, int col, int lane,
+__device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, const KvcTilePos &pos, const KvcTablePlan &pl, int lane,
                                                    const KvcRaw<REP, KvcGeom<KIND>::SLOTS, KvcGeom<KIND>::XW> &raw,
                                                    uint32_t *btab, uint32_t *mstab, float (&bias)[REP], float &unscale,
-                                                   int &sel_out, bool &lo_used)
+                                                   int &sel_out, KvcTableState &st)
 {
     constexpr int SLOTS = KvcGeom<KIND>::SLOTS;
     constexpr int NM = kvc_mfma_sets(REP);
     using T = KvcMfmaTables<REP>;
     const int D = a.head_dim;
+    const int row = pos.row;
     float bias_s[SLOTS][REP];
     float v[SLOTS][REP][2];
-    const bool straddles = SLOTS == 2 && (col * KVC_WAVE) % D + KVC_WAVE > D;      // wave-uniform
     const bool live = KIND != 0 || 2 * lane < D;
-    const int pmode = kvc_pair_mode<KIND>(a);
+    const int pmode0 = kvc_pair_mode<KIND>(a);
+    // (the second head's parameters are always held as one word of scales and one of minima: copies of the first
+    // head's where they are per token, fetched late and packed by the kernel otherwise)
+    auto pmode_of = [&](int s) { return s == 0 ? pmode0 : (int)KVC_PAIR_ADJACENT; };
+    int sel = 0;
+    if (SLOTS == 2) sel = (pos.d0 + lane) >= D;                               // 1 past a head boundary
+    sel_out = sel;
+    auto slot_of = [&](int s) { return s == 0 ? pl.slot0 : 1 - pl.slot0; };   // table slot of the tile's head s
     // Rounded mode without the softmax: the weights are the caller's fp16 values (q, or p).  Unless one of them is
     // subnormal they are their own high parts and the low parts are zero: the words go to the table as they were
     // loaded, and the low columns stay (or are made) zero.
@@ -157,7 +232,7 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
         bool subnormal = false;
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
-            if (s == 1 && !straddles) continue;
+            if (!((pl.build >> s) & 1)) continue;
 #pragma unroll
             for (int r = 0; r < REP; r++) {
                 const kvc_h2 w = __builtin_bit_cast(kvc_h2, raw.x[s][r][0]);
@@ -166,38 +241,38 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
         }
         if (!__any(live && subnormal)) {
             const int g = lane >> 1, odd = lane & 1;
-            if (live) {
 #pragma unroll
-                for (int s = 0; s < SLOTS; s++) {
-                    uint32_t *bg = btab + s * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
-                    if (lo_used) {                             // low parts an earlier tile of this wave left, in either slot
+            for (int s = 0; s < SLOTS; s++) {
+                if (!((pl.build >> s) & 1)) continue;
+                const int ts = slot_of(s);
+                if (live) {
+                    uint32_t *bg = btab + ts * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
+                    if (st.lo(ts)) {                           // low parts an earlier tile of this wave left there
 #pragma unroll
                         for (int r = 0; r < REP; r++) bg[(((2 * r + 1) >> 2) * 4 + ((2 * r + 1) & 3)) * 2] = 0u;
                     }
-                    if (s == 1 && !straddles) continue;
 #pragma unroll
                     for (int r = 0; r < REP; r++) bg[(((2 * r) >> 2) * 4 + ((2 * r) & 3)) * 2] = raw.x[s][r][0];
-                    uint32_t *mg = mstab + s * T::MSTAB_SLOT_WORDS + g * 4 + odd;
-                    kvc_mfma_min_scale_words(raw, s, pmode, mg[0], mg[2]);
+                    uint32_t *mg = mstab + ts * T::MSTAB_SLOT_WORDS + g * 4 + odd;
+                    kvc_mfma_min_scale_words(raw, s, pmode_of(s), mg[0], mg[2]);
                 }
+                st.set_lo(ts, 0);
             }
-            lo_used = false;
             unscale = 1.f;
-            int sel = 0;
-            if (SLOTS == 2) sel = ((col * KVC_WAVE) % D + lane) >= D;
-            sel_out = sel;
 #pragma unroll
             for (int r = 0; r < REP; r++) bias[r] = 0.f;
             return;
         }
     }
-    lo_used = true;
     float vmax = 0.f;
 #pragma unroll
     for (int s = 0; s < SLOTS; s++) {
 #pragma unroll
         for (int r = 0; r < REP; r++) bias_s[s][r] = 0.f, v[s][r][0] = v[s][r][1] = 0.f;
-        if (s == 1 && !straddles) continue;                    // no lane of this tile belongs to a second head
+        if (!((pl.build >> s) & 1)) continue;                  // no lane of this tile belongs to a second head, or the head's tables are there
+        st.set_lo(slot_of(s), 1);
+        int hb = pos.b, hh = pos.h;
+        if (s == 1) kvc_second_head(a, pos, hb, hh);
 #pragma unroll
         for (int r = 0; r < REP; r++) {
             float w0, w1;                                      // the two elements' weights: q, p, or exp(score - max)
@@ -209,11 +284,7 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
                 w1 = __expf(s1 - m);
                 const float l = kvc_wave_sum_dpp(w0 + w1);
                 if (lane == 0) {
-                    int bh = (col * KVC_WAVE) / D + s;
-                    const int bh_max = a.batch * a.kv_heads - 1;
-                    bh = bh < bh_max ? bh : bh_max;
-                    const int b = bh / a.kv_heads, h = bh - b * a.kv_heads;
-                    float *ml = a.ml + (((int64_t)row * a.batch + b) * a.q_heads + h * REP + r) * 2;
+                    float *ml = a.ml + (((int64_t)row * a.batch + hb) * a.q_heads + hh * REP + r) * 2;
                     ml[0] = m;     // tiles that share a head write the same pair
                     ml[1] = l;
                 }
@@ -225,11 +296,11 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
                 v[s][r][0] = w0;
                 v[s][r][1] = w1;
             } else {
-                const float sc0 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 0, pmode)) : 0.f;
-                const float sc1 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 1, pmode)) : 0.f;
+                const float sc0 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 0, pmode_of(s))) : 0.f;
+                const float sc1 = live ? kvc_half_bits_to_float(raw.scale_bits(s, 1, pmode_of(s))) : 0.f;
                 v[s][r][0] = sc0 * w0;
                 v[s][r][1] = sc1 * w1;
-                bias_s[s][r] = (float)raw.min_int(s, 0, pmode) * v[s][r][0] + (float)raw.min_int(s, 1, pmode) * v[s][r][1];
+                bias_s[s][r] = (float)raw.min_int(s, 0, pmode_of(s)) * v[s][r][0] + (float)raw.min_int(s, 1, pmode_of(s)) * v[s][r][1];
                 vmax = fmaxf(vmax, fmaxf(fabsf(v[s][r][0]), fabsf(v[s][r][1])));
             }
         }
@@ -254,26 +325,24 @@ __device__ __forceinline__ void kvc_mfma_stage_ops(const KvcFusedArgs &a, int ro
     if (live) {
 #pragma unroll
         for (int s = 0; s < SLOTS; s++) {
-            if (s == 1 && !straddles) continue;
+            if (!((pl.build >> s) & 1)) continue;
+            const int ts = slot_of(s);
 #pragma unroll
             for (int r = 0; r < REP; r++) {
                 float h0, l0, h1, l1;
                 kvc_split_weight(v[s][r][0] * down, h0, l0);
                 kvc_split_weight(v[s][r][1] * down, h1, l1);
                 const int c_hi = 2 * r, c_lo = 2 * r + 1;
-                uint32_t *bg = btab + s * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
+                uint32_t *bg = btab + ts * T::BTAB_SLOT_WORDS + g * (NM * 8) + odd;
                 bg[((c_hi >> 2) * 4 + (c_hi & 3)) * 2] = kvc_half_pair(h0, h1);
                 bg[((c_lo >> 2) * 4 + (c_lo & 3)) * 2] = kvc_half_pair(l0, l1);
             }
             if (ROUNDED) {
-                uint32_t *mg = mstab + s * T::MSTAB_SLOT_WORDS + g * 4 + odd;
-                kvc_mfma_min_scale_words(raw, s, pmode, mg[0], mg[2]);
+                uint32_t *mg = mstab + ts * T::MSTAB_SLOT_WORDS + g * 4 + odd;
+                kvc_mfma_min_scale_words(raw, s, pmode_of(s), mg[0], mg[2]);
             }
         }
     }
-    int sel = 0;
-    if (SLOTS == 2) sel = ((col * KVC_WAVE) % D + lane) >= D;                 // 1 past a head boundary
-    sel_out = sel;
 #pragma unroll
     for (int r = 0; r < REP; r++) bias[r] = (SLOTS == 2 && sel) ? bias_s[SLOTS - 1][r] : bias_s[0][r];
 }
@@ -546,43 +615,64 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
 
     if (ntiles <= 0) return;
     KvcRaw<REP, SLOTS, KvcGeom<KIND>::XW> raw;
-    kvc_fetch_tile<REP, KIND>(a, row, col, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    // (the one place where the tile's batch entry, head and channel offset are worked out by division)
+    KvcTilePos pos = kvc_tile_pos<IS_K>(a, row, col);
+    KvcTableState tabs;
+    tabs.head0 = tabs.head1 = tabs.row = -1;
+    tabs.lo0 = tabs.lo1 = 0;                                             // (the low-part columns start as zeros)
+    KvcTablePlan plan = kvc_plan_tables<KIND, ROUNDED>(a, pos, tabs);
+    kvc_fetch_tile<REP, KIND, 0, SLOTS == 2>(a, pos, __builtin_amdgcn_readlane(bi_off, 0), __builtin_amdgcn_readlane(bi_bn, 0), lane, raw);
+    // the second head's parameters where every token has groups of its own per batch entry or head: fetched only now
+    auto late_params = [&](const KvcFusedArgs &a, const KvcTilePos &p, const KvcTablePlan &pl, int lane) {
+        if constexpr (SLOTS == 2) {
+            if ((pl.build & 2) && kvc_pair_mode<KIND>(a) != KVC_PAIR_ADJACENT) {
+                int b2, h2;
+                kvc_second_head(a, p, b2, h2);
+                kvc_fetch_separate_params(a, p.row, b2, h2, lane, 1, raw);
+                // ... and kept in the form of parameters that lie next to each other: two registers instead of four
+                raw.scw[1][0] = (raw.scw[1][0] & 0xffffu) | (raw.scw[1][1] << 16);
+                raw.mnw[1][0] = (raw.mnw[1][0] & 0xffu) | ((raw.mnw[1][1] & 0xffu) << 8);
+            }
+        }
+    };
+    late_params(a, pos, plan, lane);
     float bias[REP], unscale;
     int sel = 0;
-    bool lo_used = false;          // wave-uniform: the low-part columns of the operand table hold something (they start as zeros)
     uint32_t first, longest;
     KvcStaged st = kvc_stage_payload(a, lane, raw, pack, first, longest);
     if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;       // one or two bits before the lane's first code
-    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row, col, lane, raw, btab, mstab, bias, unscale, sel, lo_used);
+    kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, pos, plan, lane, raw, btab, mstab, bias, unscale, sel, tabs);
     kvc_wave_sync();
     for (int it = 0; it < ntiles; it++) {
         // the arguments are read again per tile rather than kept in scalar registers through the decode loops (the
         // kernel needs more scalars than there are registers, and every spilled one costs a vector instruction)
         const KvcFusedArgs &a = kvc_kernarg_again<KvcFusedArgs>();
         const bool more = it + 1 < ntiles;
-        int row_next = row, col_next = col + 1;        // row-major successor
-        if (col_next == cols) col_next = 0, row_next = row + 1;
+        const KvcTilePos pos_next = kvc_tile_after<IS_K>(a, pos);          // row-major successor
+        // which of the wave's operand tables the next tile can use as they are: it then needs no weights
+        KvcTablePlan plan_next = plan;
+        if (more) plan_next = kvc_plan_tables<KIND, ROUNDED>(a, pos_next, tabs);
         // the lane number is made opaque per tile, so that the addresses the fetch and the staging derive from it
         // are not kept in registers through the decode loops
         int lane_f = lane;
         asm volatile("" : "+v"(lane_f));
         if (more)   // loads for the next tile fly while this one is decoded
-            kvc_fetch_tile<REP, KIND>(a, row_next, col_next, __builtin_amdgcn_readlane(bi_off, it + 1),
-                                      __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw);
-        const uint32_t *my_btab = btab + sel * T::BTAB_SLOT_WORDS, *my_mstab = mstab + sel * T::MSTAB_SLOT_WORDS;
+            kvc_fetch_tile<REP, KIND, 0, SLOTS == 2>(a, pos_next, __builtin_amdgcn_readlane(bi_off, it + 1),
+                                                     __builtin_amdgcn_readlane(bi_bn, it + 1), lane_f, raw, ~plan_next.build);
+        const int my_slot = sel ? 1 - plan.slot0 : plan.slot0;
+        const uint32_t *my_btab = btab + my_slot * T::BTAB_SLOT_WORDS, *my_mstab = mstab + my_slot * T::MSTAB_SLOT_WORDS;
+        // (wave-uniform: some low-part column of the tables this tile reads holds something)
+        bool lo_used = tabs.lo(plan.slot0) != 0;
+        if constexpr (SLOTS == 2) lo_used = lo_used || (plan.straddles && tabs.lo(1 - plan.slot0) != 0);
         // geometry of the results
         int64_t out_base, out_step;
         if (IS_K) {
-            const int b = col / a.kv_heads, h = col - b * a.kv_heads;
-            out_base = ((int64_t)b * a.q_heads + h * REP) * a.out_stride + (int64_t)row * KVC_WAVE;
+            out_base = ((int64_t)pos.b * a.q_heads + pos.h * REP) * a.out_stride + (int64_t)pos.row * KVC_WAVE;
             out_step = a.out_stride;
         } else {
-            const int c0 = col * KVC_WAVE;
-            const int bh0 = c0 / D, d0 = c0 - bh0 * D;                  // wave-uniform
-            const int b0 = bh0 / a.kv_heads, h0 = bh0 - b0 * a.kv_heads;
-            const int wrap = (h0 + sel == a.kv_heads) ? 1 : 0;          // the next head may open the next batch entry
-            const int b = b0 + wrap, h = wrap ? 0 : h0 + sel;
-            out_base = (((int64_t)row * a.batch + b) * a.q_heads + h * REP) * D + (d0 - sel * D);
+            int b = pos.b, h = pos.h;
+            if (sel) kvc_second_head(a, pos, b, h);                     // the next head may open the next batch entry
+            out_base = (((int64_t)pos.row * a.batch + b) * a.q_heads + h * REP) * D + (pos.d0 - sel * D);
             out_step = D;
         }
         if (fast_book && st.fits) {
@@ -664,11 +754,12 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             asm volatile("" : "+v"(lane_s));
             st = kvc_stage_payload(a, lane_s, raw, pack, first, longest);
             if (st.fits) st.u0 = 32u * KVC_PACK_LEAD + first * 8u - lead_bits;
-            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, row_next, col_next, lane_s, raw, btab, mstab, bias, unscale, sel, lo_used);
+            late_params(a, pos_next, plan_next, lane_s);
+            kvc_mfma_stage_ops<REP, KIND, ROUNDED>(a, pos_next, plan_next, lane_s, raw, btab, mstab, bias, unscale, sel, tabs);
             kvc_wave_sync();
         }
-        row = row_next;
-        col = col_next;
+        pos = pos_next;
+        plan = plan_next;
     }
 }
 

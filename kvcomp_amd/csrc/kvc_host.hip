@@ -59,6 +59,8 @@ const OptionDef g_option_defs[KVC_OPT_COUNT] = {
     {"encode_one_pass", "KVCOMP_ENCODE_ONE_PASS", 1},            // tile encoder: 1: one pass (a wave counts, places by a look-back over the tiles before it, and emits its tiles); 0: two passes; 2 / 3: one pass with one / two tiles per wave
     {"fused_half_table", "KVCOMP_FUSED_HALF_TABLE", 1},          // matrix-core kernels: two-byte decode table entries for codes of 6 or 7 bits (one LDS word per bank)
     {"encode_lookback_polls", "KVCOMP_ENCODE_LOOKBACK_POLLS", 1 << 18},   // one-pass encoder: looks that may find a word not ready before a wave gives up (some tenths of a second); -1: treat every call as given up
+    {"fused_schedule_v", "KVCOMP_FUSED_SCHEDULE_V", -1},         // the same for V launches: -1 follow fused_schedule (default schedule: runs that cover whole heads)
+    {"fused_tiles_per_wave_v", "KVCOMP_FUSED_TILES_PER_WAVE_V", -1},   // plain grid, V launches: -1 follow fused_tiles_per_wave (default: the tiles of one head or head pair)
 };
 std::atomic<int> g_options[KVC_OPT_COUNT];
 std::once_flag g_options_once;
