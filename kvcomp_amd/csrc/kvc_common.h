@@ -163,6 +163,18 @@ __device__ __forceinline__ uint32_t kvc_wave_max_dpp(uint32_t v)
     return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
 }
 
+// The kernel's argument block read again from the kernarg segment (scalar loads that hit the scalar cache): what a
+// stretch of code needs of it is then live only where it is used, not in scalar registers through everything between
+// (a kernel that needs more scalars than there are registers keeps the surplus in lanes of a vector register, and every
+// access to those costs a vector instruction).
+template <class T>
+__device__ __forceinline__ const T &kvc_kernarg_again()
+{
+    auto p = __builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(p));
+    return *(const T *)p;
+}
+
 // inclusive prefix sum over the 64 lanes of a wave
 __device__ __forceinline__ uint32_t kvc_wave_inclusive_scan(uint32_t v, int lane)
 {

@@ -1095,7 +1095,6 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
         __syncthreads();
     }
     const bool short_codes = *my_short != 0u;              // wave-uniform
-    const int nd = a.e.vec_len >> 2;
     uint64_t *bi64 = reinterpret_cast<uint64_t *>(a.e.block_infos);
     const uint32_t base = a.e.status[KVC_ONCE_BASE_WORD];
     uint32_t err = 0, max_tile = 0, longest = 0, next_off = 0;
@@ -1112,6 +1111,12 @@ __global__ void __launch_bounds__(KVC_WG, 3) kvc_encode_once_kernel(KvcStoreArgs
         // is then worked out where it is used instead of being kept in registers across the whole loop body)
         int lane = tid & 63;
         asm volatile("" : "+v"(lane));
+        // (and the arguments are read again per tile rather than kept in scalar registers through everything; so is the
+        // word count of a vector, or the 32 comparisons "word j belongs to the vector" would be worked out once for the
+        // whole kernel and kept as 32 lane masks, most of them spilled)
+        const KvcStoreArgs &a = kvc_kernarg_again<KvcStoreArgs>();
+        int nd = a.e.vec_len >> 2;
+        asm volatile("" : "+s"(nd));
         uint32_t v[32];
         if constexpr (FRONT == 1) {
             // the loads of the run's second tile are on their way while the first is counted and packed

@@ -82,16 +82,6 @@ __device__ __forceinline__ uint32_t kvc_dequant_pair(uint32_t x, uint32_t mn, ui
 // upper halves of two table entries side by side: {a >> 16, b >> 16 << 16}
 __device__ __forceinline__ uint32_t kvc_pack_hi16(uint32_t a, uint32_t b) { return __builtin_amdgcn_perm(b, a, 0x07060302u); }
 
-// The kernel's argument block read again from the kernarg segment (scalar loads that hit the scalar cache): what a
-// tile needs of it is then live only where it is used, not in scalar registers through the decode loops.
-template <class T>
-__device__ __forceinline__ const T &kvc_kernarg_again()
-{
-    auto p = __builtin_amdgcn_kernarg_segment_ptr();
-    asm volatile("" : "+s"(p));
-    return *(const T *)p;
-}
-
 // -- operand tables -----------------------------------------------------------------------------------
 // btab  [slot][group g][set][column j][element k]  fp16: weight part of element 4 g + k for column 4 set + j;
 //       column 2 r is the high part of query head r's weight, column 2 r + 1 its low part times 4096
