@@ -1,9 +1,12 @@
 """Build libkvcomp_hip.so for gfx950 with hipcc (cross-compiles without a GPU).
 
-    python -m kvcomp_amd.build            # compile every csrc/*.hip, link kvcomp_amd/lib/libkvcomp_hip.so
+    python -m kvcomp_amd.build            # compile every csrc/*.hip, link kvcomp_amd/lib/libkvcomp_hip.so,
+                                          # then the compiled `kvcomp_cuda` module over it (kvcomp_amd/ext/)
 
 Objects are compiled in parallel (one hipcc process per source file) and linked into one shared
-library that exports the C ABI declared in include/kvcomp_hip.h.
+library that exports the C ABI declared in include/kvcomp_hip.h.  The Python extension module
+(csrc/kvcomp_cuda_module.cpp, host C++ only) is compiled with g++ against the installed libtorch and
+linked to that library.
 """
 import json
 import os
@@ -16,6 +19,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 LIBPATH = os.path.join(LIBDIR, "libkvcomp_hip.so")
+EXTDIR = os.path.join(HERE, "ext")
+MODULE_SRC = os.path.join(CSRC, "kvcomp_cuda_module.cpp")
+MODULE_PATH = os.path.join(EXTDIR, "kvcomp_cuda.so")         # `import kvcomp_cuda` with EXTDIR on sys.path
 ARCH = "gfx950"
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -84,6 +90,30 @@ def build(verbose=True, jobs=None):
     return LIBPATH
 
 
+def build_module(verbose=True):
+    """The reference's `kvcomp_cuda` extension module (kvcomp_cuda_extension/export_kvcomp.cpp:8-26) over the C ABI."""
+    import sysconfig
+    import torch
+    from torch.utils.cpp_extension import include_paths
+    os.makedirs(EXTDIR, exist_ok=True)
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-w",
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+           "-I" + os.path.join(os.path.dirname(HERE), "include"), "-I" + os.path.join(rocm, "include"),
+           "-I" + sysconfig.get_paths()["include"]]
+    cmd += ["-I" + p for p in include_paths()]
+    cmd += ["-o", MODULE_PATH, MODULE_SRC, "-L" + LIBDIR, "-lkvcomp_hip", "-Wl,-rpath,$ORIGIN/../lib",
+            "-L" + torch_lib, "-Wl,-rpath," + torch_lib, "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_python"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+    return MODULE_PATH
+
+
 if __name__ == "__main__":
     build(verbose="-q" not in sys.argv)
     print("built", LIBPATH)
+    build_module(verbose="-q" not in sys.argv)
+    print("built", MODULE_PATH)
