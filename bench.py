@@ -256,19 +256,21 @@ def run_decode_loop(args, emit=True):
                                                        64, 128, 64, 128, cfg["eb_k"], cfg["eb_v"])
     log("[bench] %s" % cfg["desc"])
     layers = []
-    t0 = time.perf_counter()
+    t_prefill = 0.0                              # the stores alone: the inputs are generated on the host, layer by layer
     for l in range(L):
         k, v = make_kv(cfg, dev, seed_offset=l)
         kctx, vctx = KVCompCtx(True, B, H, D, cfg["eb_k"]), KVCompCtx(False, B, H, D, cfg["eb_v"])
         for c in (kctx, vctx):                   # as the model-facing caches set their contexts up
             c.codebook_smoothing = True          # later tokens may quantize to symbols the prompt never produced
             c.async_store = not args.sync_store  # blocks that leave the tail are encoded without waiting for the device
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
         kctx.store(k, want_symbols=False)
         vctx.store(v, want_symbols=False)
+        torch.cuda.synchronize()
+        t_prefill += time.perf_counter() - t0
         layers.append((kctx, vctx, A.CompressedAttention(kctx, vctx)))
         del k, v
-    torch.cuda.synchronize()
-    t_prefill = time.perf_counter() - t0
     g = torch.Generator(device=dev).manual_seed(1236)
     new_k = torch.randn(L, 1, B, H, D, generator=g, device=dev).to(torch.float16)
     new_v = torch.randn(L, 1, B, H, D, generator=g, device=dev).to(torch.float16)

@@ -93,6 +93,17 @@ int kvc_abi_version(void);
  *                           block_infos is not 8-byte aligned or the call has more than 84 224 tiles, and by the other
  *                           encoders that start from uint8 symbols; 2 / 3: one pass for every encoder, with
  *                           always one / two tiles per wave.  Same bytes either way.
+ *   "encode_lookback_polls": how often a wave of the one-pass encoder asks again for a size that an earlier tile has not
+ *                           published yet before it gives the call up (default 262144; a wave normally asks 50 - 60
+ *                           times at most, reported in d_result[6]).  Workgroups take their tiles by a ticket drawn when
+ *                           they start, so what a wave waits for has always started before it; a call that is given up
+ *                           all the same is encoded again by one workgroup in two passes inside the same launch
+ *                           sequence (same bytes, no error, 50 - 100 x slower).  0: every wait gives up at once, -1:
+ *                           every call is treated as given up -- both only drive that path from a test.
+ *   "fused_schedule_v", "fused_tiles_per_wave_v": -1 (default): as "fused_schedule" / "fused_tiles_per_wave"; other
+ *                           values apply to the V kernels only (whose runs follow the head pattern: a run of the
+ *                           default schedule is a multiple of lcm(head_dim, 64) / 64 tiles, so that the tiles of a run
+ *                           share their heads' operand tables).
  *   "attention_tail_in_merge": 1 (default): kvc_attention_decode handles V's fp16 tail (up to 1024 tokens, K compressed
  *                           at least as far as V) inside its merge kernel; 0: with two kernels of its own.
  *   "decode_pipelined":      1 (default): plain decode and decode + dequantize run on the fused kernels' tile
@@ -186,7 +197,13 @@ int kvc_store_fused(int is_k, const void *d_x_f16, int64_t tokens, int64_t batch
  *   d_result    device uint32[8], zeroed once by the caller, then shared by successive calls:
  *               [0] payload bytes of the latest call, [1] error bits of all calls so far (0 = none), [2] largest tile
  *               payload and [3] longest lane stream so far (sizing hints of the fused decoders), [4] tiles encoded
- *               so far, [5] block_info.offset of the latest call's first tile.
+ *               so far, [5] block_info.offset of the latest call's first tile, [6] the most look-back polls any wave of
+ *               any one-pass call so far needed (see "encode_lookback_polls"), [7] reserved.
+ * Scratch memory: encodes, the fused matvecs and kvc_attention_decode take 16 KiB slots of a per-device pool, handed out
+ * in turn per call (32 slots) -- except under stream capture (hipStreamIsCapturing), where every recorded call gets a
+ * slot of its own that is never handed out again (480 such slots per device; beyond them the call fails with a
+ * message), so replays of a graph never share scratch memory with later eager calls.  The pool is allocated by the
+ * first call on a device, which therefore must not be a recorded one.
  * kvc_encode_result copies d_result to the host (it waits for the stream), turns error bits into an error return
  * and hands out the figures (any pointer may be NULL). */
 typedef struct kvc_encode_job {
