@@ -915,7 +915,7 @@ constexpr int KVC_DEFAULT_SCHEDULE_UNIT3 = 67020; // runs of 6 (two head pairs o
 // `unit`: V tiles (matrix-core kernels, rounded arithmetic) after which the heads repeat -- the tiles of one head, or of
 // a pair of heads where head_dim is no multiple of 64 (three tiles over two heads of 96 channels): a wave that takes
 // whole units builds every head's operand tables once.  0: nothing to share (K tiles; the other kernels).
-static int kvc_plan_tiles_per_wave(int64_t tiles, int unit = 0)
+static int kvc_plan_tiles_per_wave(int64_t tiles, int unit = 0, int rep = 1)
 {
     const int forced_v = unit ? kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE_V) : -1;
     const int forced = forced_v > 0 ? forced_v : kvc_option(KVC_OPT_FUSED_TILES_PER_WAVE);
@@ -923,7 +923,9 @@ static int kvc_plan_tiles_per_wave(int64_t tiles, int unit = 0)
     // measured on MI355X: two is best once there are enough tiles (the fetch of the second overlaps the
     // decode of the first; 49 152 tiles: 3 % faster than one); at 16 384 tiles one is 3 % faster, and longer runs
     // only leave fewer workgroups to balance over the chip (8 per wave: 15 % slower)
-    if (unit > 1 && unit <= 4 && forced_v < 0 && tiles >= 8192) return unit;
+    // (V, 16 384 tiles of head_dim 128: with four query heads per KV head, whose four softmaxes and operand tables two
+    // tiles of a head then share, 49.1 us for two per wave against 50.4 for one; with one query head 40.1 against 37.6)
+    if (unit > 1 && unit <= 4 && forced_v < 0 && tiles >= 8192 && (rep >= 4 || tiles >= 32768)) return unit;
     return tiles >= 32768 ? 2 : 1;
 }
 
@@ -1056,7 +1058,7 @@ static int kvc_fused(int is_k, const uint8_t *d_decode_tree, int64_t decode_tree
         while (l % KVC_WAVE != 0) l += head_dim;               // least common multiple of head_dim and 64
         unit = (int)(l / KVC_WAVE);
     }
-    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols, unit);
+    a.s.tiles_per_wave = kvc_plan_tiles_per_wave(rows * a.s.cols, unit, (int)rep);
     KvcTimer timer(elapsed_ms, stream);
     if (!d_luts) {
         if (int rc = kvc_launch_build_lut(d_decode_tree, decode_tree_bytes, tree_format, (uint32_t *)slot, 1, 0, stream)) return rc;
