@@ -24,7 +24,9 @@ DEV = "cuda:0"
 @pytest.fixture(scope="module")
 def ext():
     from kvcomp_amd import build
-    assert os.path.exists(build.MODULE_PATH), "kvcomp_amd/ext/kvcomp_cuda.so is not built: run python -m kvcomp_amd.build"
+    if not os.path.exists(build.MODULE_PATH):          # normally built beforehand (python -m kvcomp_amd.build)
+        assert os.path.exists(build.LIBPATH), "libkvcomp_hip.so is not built: run python -m kvcomp_amd.build"
+        build.build_module(verbose=False)
     spec = importlib.util.spec_from_file_location("kvcomp_cuda", build.MODULE_PATH)
     mod = importlib.util.module_from_spec(spec)
     spec.loader.exec_module(mod)
