@@ -449,7 +449,7 @@ def other_configs(args):
 
 
 def run_model_decode(args, emit=True):
-    """cfg4 as BASELINE.json words it: the Llama-2-7B architecture with random-init fp16 weights (stock `transformers`
+    """cfg4 as the headline configuration list words it: the Llama-2-7B architecture with random-init fp16 weights (stock `transformers`
     modelling code), a compressed KV cache in every layer, batch 8, a 4096-token random prompt and greedy generation;
     single-token steps attend on the compressed form through the "kvcomp" attention implementation.  Tokens are random,
     so the text means nothing; the arithmetic and the memory traffic are those of the real model."""
