@@ -73,7 +73,10 @@ constexpr int kvc_fused_mfma_occupancy(int rep, int kind)
 {
     // (four query heads, K: the kernel needs 80 registers, which leave six waves; with a bound of five the register
     // allocator settles on 81 and the sixth wave is lost: 46 -> 49 us at batch 16 x 8 KV heads x 8192 tokens)
-    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : KVC_MFMA_OCC_V1) : (rep == 4 && kind == 0) ? 6 : kvc_fused_occupancy(rep, kind);
+    // (one query head, V tiles of one head each -- head_dim a multiple of 64 --: 65 registers, seven waves, 37.7 -> 36.6 us
+    // at batch 8 x 32 heads x 128 x 4096 tokens; the kernels for tiles that straddle two heads need 77 and spill at 72)
+    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : (kind == 1 || kind == 3) ? KVC_MFMA_OCC_V1 + 1 : KVC_MFMA_OCC_V1)
+                    : (rep == 4 && kind == 0) ? 6 : kvc_fused_occupancy(rep, kind);
 }
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
 constexpr int KVC_PACK_LEAD = 4;      // zero words in front of the packed payload: bit positions never drop below 2

@@ -693,7 +693,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             else run(std::false_type{});
             // register i of lane 4 b + j: row 4 b + i, column 4 set + j; the even columns take their low parts from
             // the lane to their right and carry the results of query head 2 set + j / 2
-            const int j = lane & 3, rows4 = (lane >> 2) * 4;
+            int lane_e = lane;
+            // (one query head: nothing derived from the lane number is kept across the decode loops, which lets the
+            // single-head V kernel fit the registers of seven waves; with more heads the kernels measured no better for it)
+            if constexpr (REP == 1) asm volatile("" : "+v"(lane_e));
+            const int j = lane_e & 3, rows4 = (lane_e >> 2) * 4;
 #pragma unroll
             for (int s = 0; s < NM; s++) {
                 float res[4];
@@ -730,9 +734,11 @@ __global__ void __launch_bounds__(KVC_WG, kvc_fused_mfma_occupancy(REP, KIND)) k
             else
                 res = kvc_mfma_slow_tile<REP, true, ROUNDED>(st.gwords, st.gnwords, st.gpos, lut_g, n, my_btab, my_mstab, 0u);
             // here a lane holds the results of its own row; in a V tile every lane's head slot is its block's
+            int lane_o = lane;
+            if constexpr (REP == 1) asm volatile("" : "+v"(lane_o));
 #pragma unroll
             for (int r = 0; r < REP; r++) {
-                const int64_t o = out_base + r * out_step + lane;
+                const int64_t o = out_base + r * out_step + lane_o;
                 const float v = res.v[r] * unscale + bias[r];
                 if (a.out_f32) reinterpret_cast<float *>(a.out)[o] = v;
                 else reinterpret_cast<__half *>(a.out)[o] = __float2half(v);
