@@ -73,9 +73,11 @@ constexpr int kvc_fused_mfma_occupancy(int rep, int kind)
 {
     // (four query heads, K: the kernel needs 80 registers, which leave six waves; with a bound of five the register
     // allocator settles on 81 and the sixth wave is lost: 46 -> 49 us at batch 16 x 8 KV heads x 8192 tokens)
-    // (one query head, V tiles of one head each -- head_dim a multiple of 64 --: 65 registers, seven waves, 37.7 -> 36.6 us
-    // at batch 8 x 32 heads x 128 x 4096 tokens; the kernels for tiles that straddle two heads need 77 and spill at 72)
-    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : (kind == 1 || kind == 3) ? KVC_MFMA_OCC_V1 + 1 : KVC_MFMA_OCC_V1)
+    // (one query head, V: seven waves.  Tiles of one head each -- head_dim a multiple of 64 --: 65 registers, 37.7 -> 36.4 us
+    // at batch 8 x 32 heads x 128 x 4096 tokens; eight waves fit too, with 30 spilled scalars, and measured no better.
+    // Tiles that may straddle two heads, softmax on the fly: 72 registers without a spill only in a translation unit of
+    // its own, kvc_fused_mfma_v96.hip; 71.7 -> 68.4 us at batch 4 x 32 heads x 96 x 32 768 tokens.)
+    return rep == 1 ? (kind == 0 ? KVC_MFMA_OCC_K1 : (kind == 1 || kind == 3 || kind == 4) ? KVC_MFMA_OCC_V1 + 1 : KVC_MFMA_OCC_V1)
                     : (rep == 4 && kind == 0) ? 6 : kvc_fused_occupancy(rep, kind);
 }
 constexpr int KVC_PRE_CHUNKS = 4;     // 16-byte chunks per lane fetched one tile ahead (4 KiB of payload)
