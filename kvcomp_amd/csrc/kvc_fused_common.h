@@ -1,5 +1,5 @@
 // kvc_fused_common.h -- pieces shared by the fused decode + matvec kernels (kvc_fused.hip: fp32 FMA loops and plain
-// decode; kvc_fused_mfma.hip: matrix-core loops): launch arguments, the one-tile-ahead fetch, payload staging.
+// decode; kvc_fused_mfma_impl.h: matrix-core loops): launch arguments, the one-tile-ahead fetch, payload staging.
 #pragma once
 #include "kvc_tile.h"
 
@@ -472,7 +472,7 @@ __device__ __forceinline__ KvcStaged kvc_stage_payload(const KvcFusedArgs &a, in
 }
 
 // ---------------------------------------------------------------------------------------------------
-// matrix-core variant (kvc_fused_mfma.hip)
+// matrix-core variant (kvc_fused_mfma_impl.h)
 // ---------------------------------------------------------------------------------------------------
 // Columns of the operand matrix: every query head contributes a high and a low fp16 part of its weight, four
 // columns per v_mfma_f32_4x4x4_16b_f16.
