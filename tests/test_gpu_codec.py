@@ -311,6 +311,45 @@ def test_errors_raise_instead_of_aborting():
         m.build_codebook([torch.zeros(100, dtype=torch.uint8, device=DEV)])   # a lone symbol has no usable code
 
 
+@pytest.mark.parametrize("binding", ["ctypes", "compiled"])
+@pytest.mark.parametrize("is_k", [True, False])
+def test_empty_inputs_are_no_ops(is_k, binding):
+    """Zero tokens: sizes are zero, the encoder returns empty views, the decoders and the fused products return without
+    touching anything (the reference would launch an empty grid and abort on the launch error)."""
+    if binding == "ctypes":
+        m = kc()
+    else:
+        import importlib.util
+        from kvcomp_amd import build
+        spec = importlib.util.spec_from_file_location("kvcomp_cuda", build.MODULE_PATH)
+        m = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(m)
+    H, D = 4, 128
+    bs = 64 if is_k else 128
+    x = S.synth_k(128, 1, H, D)
+    sym = _make_stream(x, True, 0.1, O.MASK_K_BLOCK, 64)["sym"]
+    _, enc, tree = m.build_codebook([_dev(sym)])
+    empty = torch.zeros(0, bs, 1, H, D, dtype=torch.uint8, device=DEV)
+    assert tuple(m.calculate_buffer_size(empty, is_k, H, D)) == (0, 0, 8, 0)
+    bufs = [torch.full((8,), 0xAB, dtype=torch.uint8, device=DEV) for _ in range(4)]
+    efn = m.k_entropy_encode_cuda_export if is_k else m.v_entropy_encode_cuda_export
+    payload, bi, ti = efn(empty, enc.to(DEV), bufs[0], bufs[1], bufs[2], bufs[3], 0, H, D)
+    assert payload.numel() == bi.numel() == ti.numel() == 0
+    assert all(bool((b == 0xAB).all()) for b in (bufs[0], bufs[1], bufs[3]))
+    z = torch.zeros(0, dtype=torch.uint8, device=DEV)
+    dfn = m.k_entropy_decode_cuda_export if is_k else m.v_entropy_decode_cuda_export
+    assert dfn(z, z, z, tree.to(DEV), empty, H, D) == 0.0
+    mins, scales = torch.zeros(0, dtype=torch.int8, device=DEV), torch.zeros(0, dtype=torch.float16, device=DEV)
+    if is_k:
+        out = torch.zeros(1, H, 0, dtype=torch.float16, device=DEV)
+        assert m.k_decode_and_mat_vec_mul_cuda_export(tree.to(DEV), z, z, z, mins, scales, S.synth_q(1, H, D).to(DEV), out, H, D) == 0.0
+    else:
+        p = torch.zeros(1, H, 0, dtype=torch.float16, device=DEV)
+        out = torch.zeros(0, 1, H, D, dtype=torch.float16, device=DEV)
+        assert m.v_decode_and_mat_vec_mul_cuda_export(tree.to(DEV), z, z, z, mins, scales, p, out, H, D) == 0.0
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("is_k", [True, False])
 @pytest.mark.parametrize("nsym", [14, 22])
 def test_fused_with_long_codes_uses_slow_path(is_k, nsym, fused_mode):
