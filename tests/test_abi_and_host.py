@@ -33,6 +33,25 @@ def test_library_exports_every_declared_symbol():
     assert _lib.lib().kvc_abi_version() == 2
 
 
+def test_every_tuning_option_is_documented_in_the_header_and_known_to_the_library():
+    """The option names listed in include/kvcomp_hip.h are exactly the ones kvc_get_option answers for (names are read
+    from the header's comment and from the library's option table in csrc/kvc_host.hip)."""
+    import ctypes as C
+    import re
+    from kvcomp_amd import _lib
+    header = open(os.path.join(ROOT, "include", "kvcomp_hip.h")).read()
+    block = header[header.index("Tuning knobs"):header.index("int kvc_set_option")]
+    documented = set(re.findall(r'"([a-z_0-9]+)"', block))
+    table = open(os.path.join(ROOT, "kvcomp_amd", "csrc", "kvc_host.hip")).read()
+    known = set(re.findall(r'\{"([a-z_0-9]+)", "KVCOMP_[A-Z_0-9]+",', table))
+    assert known and documented == known, (sorted(documented - known), sorted(known - documented))
+    L = _lib.lib()
+    for name in known:
+        v = C.c_int(0)
+        assert L.kvc_get_option(name.encode(), C.byref(v)) == 0, name
+    assert L.kvc_get_option(b"no_such_option", C.byref(C.c_int(0))) != 0
+
+
 def test_missing_library_fails_loudly(monkeypatch):
     from kvcomp_amd import _lib
     monkeypatch.setattr(_lib, "_LIB", None)
